@@ -1,0 +1,36 @@
+"""Builds fp6_llm_amd/libfp6mi.so (host code + gfx950 kernels + C ABI) with hipcc. Run: python -m fp6_llm_amd.build"""
+import os
+import shutil
+import subprocess
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(HERE)
+SOURCES = [os.path.join(HERE, "csrc", "fp6mi_host.cpp"), os.path.join(HERE, "csrc", "fp6mi_gemm.hip")]
+OUTPUT = os.path.join(HERE, "libfp6mi.so")
+
+
+def hipcc_path():
+    for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
+        if cand and os.path.exists(cand):
+            return cand
+    raise RuntimeError("hipcc not found; the FPx engine cannot be built without the ROCm compiler")
+
+
+def build(verbose=False):
+    """Compiles every HIP/C++ source for gfx950 into libfp6mi.so (always recompiles)."""
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+           # packed FP32 VALU forms are kept out of the generated code on this hardware pool
+           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-I" + os.path.join(ROOT, "include")] + SOURCES + ["-o", OUTPUT + ".tmp"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed building libfp6mi.so")
+    os.replace(OUTPUT + ".tmp", OUTPUT)
+    return OUTPUT
+
+
+if __name__ == "__main__":
+    print(build(verbose=True))

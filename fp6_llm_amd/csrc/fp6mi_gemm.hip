@@ -1,0 +1,465 @@
+// gfx950 (MI355X) kernels of the FPx x FP16 linear layer, their launchers and the C ABI.
+//
+// Roles taken over from the reference (usyd-fsalab/fp6_llm, paths relative to it):
+//   gemm_stream   <- QUANT_GEMM_Kernel        fp6_llm/csrc/include/kernel_matmul.cuh:29-191
+//   splitk_reduce <- SplitK_Reduction         fp6_llm/csrc/include/kernel_reduction.cuh:28-47
+//   launchers     <- fpx_linear_kernel        fp6_llm/csrc/fp6_linear.cu:44-102
+// The design is not a translation: weights use the native layout described in fp6mi_host.cpp, go from HBM straight
+// to VGPRs with 128-bit non-temporal loads, FP6 codes are converted by the CDNA4 instruction
+// v_cvt_scalef32_pk32_f16_bf6 (BF6 = e3m2, bias 3, no inf/nan: the very format of the reference), FP5 codes by
+// shift/mask into fp16 bit patterns, and v_mfma_f32_16x16x32_f16 accumulates in FP32.  The per-row scale (and the
+// 2^14 exponent rebias of FP5) is applied once to the FP32 sums instead of to every weight.
+#include <hip/hip_runtime.h>
+
+#include "fp6mi_internal.h"
+
+namespace {
+
+typedef _Float16 half_t;
+typedef _Float16 v8h __attribute__((ext_vector_type(8)));
+typedef _Float16 v32h __attribute__((ext_vector_type(32)));
+typedef float    v4f __attribute__((ext_vector_type(4)));
+typedef uint32_t v2u __attribute__((ext_vector_type(2)));
+typedef uint32_t v4u __attribute__((ext_vector_type(4)));
+typedef uint32_t v6u __attribute__((ext_vector_type(6)));
+
+constexpr int kWave = 64;
+
+template <int XB> struct Fmt;
+template <> struct Fmt<6> { static constexpr int block_bytes = 3072; static constexpr float post_scale = 1.0f; };
+template <> struct Fmt<5> { static constexpr int block_bytes = 2560; static constexpr float post_scale = 16384.0f; };
+
+// The weights of one lane for one 16x256 block, as loaded from memory.
+template <int XB> struct WFrag;
+template <> struct WFrag<6> { v4u a, b, c; };
+template <> struct WFrag<5> { v4u a, b; v2u s; };
+
+template <int XB> __device__ __forceinline__ WFrag<XB> load_wfrag(const uint8_t *block, int lane);
+template <> __device__ __forceinline__ WFrag<6> load_wfrag<6>(const uint8_t *block, int lane)
+{
+    const v4u *p = reinterpret_cast<const v4u *>(block) + lane;
+    WFrag<6>   f;
+    f.a = __builtin_nontemporal_load(p);
+    f.b = __builtin_nontemporal_load(p + 64);
+    f.c = __builtin_nontemporal_load(p + 128);
+    return f;
+}
+template <> __device__ __forceinline__ WFrag<5> load_wfrag<5>(const uint8_t *block, int lane)
+{
+    const v4u *p = reinterpret_cast<const v4u *>(block) + lane;
+    WFrag<5>   f;
+    f.a = __builtin_nontemporal_load(p);
+    f.b = __builtin_nontemporal_load(p + 64);
+    f.s = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(block + 2048) + lane);
+    return f;
+}
+
+// A operands (8 halfs = k 8q..8q+7 of this lane's row) of the eight MFMA steps of a block.
+// FP6: exact values.  FP5: values times 2^-14 (fp16 subnormals included; the MFMA does not flush them).
+template <int XB> struct AOps { v8h s[8]; };
+
+__device__ __forceinline__ v8h slice8(const v32h &v, int i)
+{
+    switch (i) {
+    case 0: return __builtin_shufflevector(v, v, 0, 1, 2, 3, 4, 5, 6, 7);
+    case 1: return __builtin_shufflevector(v, v, 8, 9, 10, 11, 12, 13, 14, 15);
+    case 2: return __builtin_shufflevector(v, v, 16, 17, 18, 19, 20, 21, 22, 23);
+    default: return __builtin_shufflevector(v, v, 24, 25, 26, 27, 28, 29, 30, 31);
+    }
+}
+
+__device__ __forceinline__ void convert(const WFrag<6> &f, AOps<6> &o)
+{
+    v6u  lo = { f.a[0], f.a[1], f.a[2], f.a[3], f.b[0], f.b[1] };
+    v6u  hi = { f.b[2], f.b[3], f.c[0], f.c[1], f.c[2], f.c[3] };
+    v32h h0 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(lo, 1.0f);
+    v32h h1 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(hi, 1.0f);
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        o.s[i]     = slice8(h0, i);
+        o.s[4 + i] = slice8(h1, i);
+    }
+}
+
+__device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
+{
+    constexpr uint32_t kNib = 0x0F000F00u, kSign = 0x80008000u;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        uint32_t w  = (s < 4) ? f.a[s & 3] : f.b[s & 3];
+        uint32_t sg = f.s[s >> 2] << (4 * (s & 3));
+        v4u      r;
+        r[0]   = (w & kNib) | (sg & kSign);
+        r[1]   = ((w << 4) & kNib) | ((sg << 1) & kSign);
+        r[2]   = ((w >> 4) & kNib) | ((sg << 2) & kSign);
+        r[3]   = ((w << 8) & kNib) | ((sg << 3) & kSign);
+        o.s[s] = __builtin_bit_cast(v8h, r);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gemm_stream: weight-bandwidth-bound GEMM for small batches.
+//   grid  = (M/16 row tiles, splitK, ceil(N / (16*NT)))      block = WAVES wavefronts
+// A workgroup owns 16 output rows and 16*NT batch columns over the K blocks of its split; its wavefronts take the
+// blocks round-robin (K is split inside the workgroup), each streaming its weights HBM -> VGPR and its slice of the
+// activations L2 -> VGPR directly in MFMA B-operand order; partial accumulators are summed through LDS.
+// ---------------------------------------------------------------------------------------------------------------
+template <int XB, int NT, int WAVES>
+__global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
+                                                            const half_t *__restrict__ X, half_t *__restrict__ C,
+                                                            float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
+                                                            uint32_t units, uint32_t splitK)
+{
+    __shared__ float red[WAVES][NT][256];
+
+    const int      lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int      col = lane & 15, q = lane >> 4;
+    const uint32_t R = blockIdx.x, split = blockIdx.y, nbase = blockIdx.z * (16 * NT);
+
+    const uint32_t avg = units / splitK, extra = units % splitK;
+    const uint32_t u0 = split * avg + (split < extra ? split : extra);
+    const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
+
+    const uint8_t *wrow = W + (size_t)R * units * Fmt<XB>::block_bytes;
+
+    v4f acc[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) acc[t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+
+    const half_t *xrow[NT];
+    bool          xok[NT];
+#pragma unroll
+    for (int t = 0; t < NT; t++) {
+        uint32_t n = nbase + 16 * t + col;
+        xok[t]     = n < N;
+        xrow[t]    = X + (size_t)(xok[t] ? n : 0) * K + 8 * q;
+    }
+
+    for (uint32_t u = u0 + wave; u < u1; u += WAVES) {
+        WFrag<XB> wf = load_wfrag<XB>(wrow + (size_t)u * Fmt<XB>::block_bytes, lane);
+        v8h       xb[8][NT];
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            uint32_t k = u * 256 + 32 * s;
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                v8h z = { 0, 0, 0, 0, 0, 0, 0, 0 };
+                xb[s][t] = (xok[t] && k + 8 * q < K) ? *reinterpret_cast<const v8h *>(xrow[t] + k) : z;
+            }
+        }
+        AOps<XB> a;
+        convert(wf, a);
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.s[s], xb[s][t], acc[t], 0, 0, 0);
+    }
+
+    // acc[t][i] = sum for output row 4q+i, batch column 16t+col
+#pragma unroll
+    for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[wave][t][lane * 4]) = acc[t];
+    __syncthreads();
+
+    for (int e = threadIdx.x; e < NT * 256; e += WAVES * kWave) {
+        int   t = e >> 8, r = e & 255, n = r >> 4, mm = r & 15;
+        int   idx = (((mm >> 2) * 16 + n) << 2) | (mm & 3);
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) sum += red[w][t][idx];
+        uint32_t ng = nbase + 16 * t + n, mg = R * 16 + mm;
+        if (ng < N) {
+            float v = sum * ((float)scales[mg] * Fmt<XB>::post_scale);
+            if (splitK == 1)
+                C[(size_t)ng * M + mg] = (half_t)v;
+            else
+                ws[((size_t)split * N + ng) * M + mg] = v;
+        }
+    }
+}
+
+// C[i] = fp16_rn(sum over splits, in split order, of ws[s][i]); four outputs per thread.
+__global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK)
+{
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= MN) return;
+    v4f sum = { 0.f, 0.f, 0.f, 0.f };
+    for (int s = 0; s < splitK; s++) sum += *reinterpret_cast<const v4f *>(ws + (size_t)s * MN + i);
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    v4h o = { (half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3] };
+    *reinterpret_cast<v4h *>(C + i) = o;
+}
+
+// Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
+template <int XB>
+__global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, const uint8_t *__restrict__ W,
+                                                     const half_t *__restrict__ scales, uint32_t M, uint32_t K, uint32_t units)
+{
+    const int      lane = threadIdx.x & 63;
+    const uint32_t blk = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= (M / 16) * units) return;
+    const uint32_t R = blk / units, U = blk % units;
+    const int      m = lane & 15, q = lane >> 4;
+    WFrag<XB>      wf = load_wfrag<XB>(W + (size_t)blk * Fmt<XB>::block_bytes, lane);
+    AOps<XB>       a;
+    convert(wf, a);
+    const half_t sc = scales[R * 16 + m], post = (half_t)Fmt<XB>::post_scale;
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        uint32_t k = U * 256 + 32 * s + 8 * q;
+        if (k < K) {
+            v8h v = a.s[s];
+            if (XB == 5) v = v * post; // exact: a power of two, results are at most 7
+            v = v * sc;                // one round-to-nearest-even, like fp16_rn(value * scale)
+            *reinterpret_cast<v8h *>(out + (size_t)(R * 16 + m) * K + k) = v;
+        }
+    }
+}
+
+// Reference layout -> native layout on the device.  One thread per (row tile, K block, lane): it gathers its 64
+// codes bit piece by bit piece from the reference's segment arrays and writes its 10 or 12 native dwords.
+__constant__ uint8_t kInvOrder4[8]  = { 4, 0, 6, 2, 5, 1, 7, 3 };
+__constant__ uint8_t kInvOrder2[16] = { 8, 0, 12, 4, 9, 1, 13, 5, 10, 2, 14, 6, 11, 3, 15, 7 };
+
+template <int XB>
+__global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restrict__ native, const uint8_t *__restrict__ ref,
+                                                             uint32_t M, uint32_t K, uint32_t units)
+{
+    const int      lane = threadIdx.x & 63;
+    const uint32_t blk = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= (M / 16) * units) return;
+    const uint32_t R = blk / units, U = blk % units;
+    const int      m = lane & 15, q = lane >> 4;
+    const uint32_t row = R * 16 + m, tile = row >> 6, block = (row >> 4) & 3, rin = row & 15, g = rin & 7, rowhalf = rin >> 3;
+    // segment arrays: FP6 = [2-bit | 4-bit], FP5 = [1-bit | 4-bit]
+    const uint32_t *seg_hi = reinterpret_cast<const uint32_t *>(ref);
+    const uint32_t *seg4   = reinterpret_cast<const uint32_t *>(ref + (size_t)M * K * (XB == 6 ? 2 : 1) / 8);
+    uint8_t         c[64];
+#pragma unroll 1
+    for (int s = 0; s < 8; s++) {
+        uint32_t k0 = U * 256 + 32 * s + 8 * q;
+        for (int j = 0; j < 8; j++) {
+            uint32_t col = k0 + j, code = 0;
+            if (col < K) {
+                uint32_t slice = col >> 4, cc = col & 15, t = (cc & 7) >> 1;
+                uint32_t el = (cc & 1) | (rowhalf << 1) | ((cc >> 3) << 2);
+                uint32_t l32 = 4 * g + t;
+                { // 4-bit piece: q4 = block, pre = el
+                    uint32_t word = seg4[((size_t)(tile * (K / 16) + slice) * 4 + block) * 32 + l32];
+                    code |= (word >> (28 - 4 * kInvOrder4[el])) & 15u;
+                }
+                if (XB == 6) { // 2-bit piece: q2 = block/2, pre = (block%2)*8 + el
+                    uint32_t word = seg_hi[((size_t)(tile * (K / 16) + slice) * 2 + (block >> 1)) * 32 + l32];
+                    code |= ((word >> (30 - 2 * kInvOrder2[(block & 1) * 8 + el])) & 3u) << 4;
+                } else { // 1-bit piece: q1 = 0, pre = block*8 + el; order_1 maps p -> pre, inverted arithmetically:
+                    // order_1[p]-1 = 4*(p%8) + {1,3,0,2}[p/8]  =>  p = 8*{2,0,3,1}[pre%4] + pre/4
+                    uint32_t pre = block * 8 + el;
+                    uint32_t p   = 8 * ((0x1302u >> (4 * (pre & 3))) & 3u) + (pre >> 2);
+                    uint32_t word = seg_hi[((size_t)(tile * (K / 16) + slice)) * 32 + l32];
+                    code |= ((word >> (31 - p)) & 1u) << 4;
+                }
+            }
+            c[8 * s + j] = (uint8_t)code;
+        }
+    }
+    uint8_t *dst = native + (size_t)blk * Fmt<XB>::block_bytes;
+    if (XB == 6) {
+        uint32_t d[12];
+        for (int h = 0; h < 2; h++) {
+            uint64_t accb = 0;
+            int      nb = 0, w = 0;
+            for (int i = 0; i < 32; i++) {
+                accb |= (uint64_t)c[32 * h + i] << nb;
+                nb += 6;
+                if (nb >= 32) { d[6 * h + w++] = (uint32_t)accb; accb >>= 32; nb -= 32; }
+            }
+        }
+        for (int i = 0; i < 3; i++) {
+            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
+            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        }
+    } else {
+        const int slot[4] = { 2, 1, 3, 0 };
+        uint32_t  d[10];
+        d[8] = d[9] = 0;
+        for (int s = 0; s < 8; s++) {
+            uint32_t word = 0;
+            for (int p = 0; p < 4; p++) {
+                uint32_t lo = c[8 * s + 2 * p], hi = c[8 * s + 2 * p + 1];
+                int      pp = 4 * (s & 3) + p;
+                word |= (lo & 15u) << (4 * slot[p]) | (hi & 15u) << (4 * (slot[p] + 4));
+                d[8 + (s >> 2)] |= ((lo >> 4) & 1u) << (15 - pp) | ((hi >> 4) & 1u) << (31 - pp);
+            }
+            d[s] = word;
+        }
+        for (int i = 0; i < 2; i++) {
+            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
+            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        }
+        v2u sv = { d[8], d[9] };
+        reinterpret_cast<v2u *>(dst + 2048)[lane] = sv;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------ launch helpers
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+template <int XB, int NT, int WAVES>
+int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+                  int splitK)
+{
+    uint32_t units = (uint32_t)((K + 255) / 256);
+    dim3     grid((uint32_t)(M / 16), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
+    hipLaunchKernelGGL((gemm_stream<XB, NT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
+                       static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M,
+                       (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
+    return (int)hipGetLastError();
+}
+
+template <int XB>
+int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
+                  int splitK)
+{
+    size_t units = (K + 255) / 256;
+    size_t per_split = (units + (size_t)splitK - 1) / (size_t)splitK;
+    int    rc;
+    if (N <= 16) {
+        if (per_split > 8) rc = launch_stream<XB, 1, 16>(st, W, sc, B, C, ws, M, N, K, splitK);
+        else if (per_split > 4) rc = launch_stream<XB, 1, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
+        else rc = launch_stream<XB, 1, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
+    } else if (N <= 32) {
+        if (per_split > 4) rc = launch_stream<XB, 2, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
+        else rc = launch_stream<XB, 2, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
+    } else {
+        if (per_split > 4) rc = launch_stream<XB, 4, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
+        else rc = launch_stream<XB, 4, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
+    }
+    if (rc != 0) return rc;
+    if (splitK > 1) {
+        size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
+        hipLaunchKernelGGL(splitk_reduce, dim3((uint32_t)((MN / 4 + 255) / 256)), dim3(256), 0, st, static_cast<half_t *>(C), ws, MN,
+                           splitK);
+        rc = (int)hipGetLastError();
+    }
+    return rc;
+}
+
+} // namespace
+
+// ------------------------------------------------------------------------------------------------ C ABI
+
+extern "C" {
+
+const char *fp6mi_error_string(int code)
+{
+    switch (code) {
+    case FP6MI_OK: return "success";
+    case FP6MI_ERR_FORMAT: return "unsupported (E,M): only FP6_e3m2 (3,2) and FP5_e2m2 (2,2)";
+    case FP6MI_ERR_SHAPE: return "unsupported shape: need M % 256 == 0 (64 for CPU packers, 16 for native packers), K % 64 == 0, N >= 1, distinct in/out";
+    case FP6MI_ERR_NULL: return "a required pointer is NULL";
+    case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
+    case FP6MI_ERR_SPLITK: return "splitK must be >= 1";
+    case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned";
+    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fp6mi error";
+    }
+}
+
+int fp6mi_version(void) { return 100; }
+
+int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
+int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }
+int fp6mi_dequant(int E, int Mb, void *out, const void *raw, size_t M, size_t K, const void *sc) { return fp6mi::dequant(E, Mb, out, raw, M, K, sc); }
+size_t fp6mi_native_bytes(int E, int Mb, size_t M, size_t K) { return fp6mi::native_bytes(E, Mb, M, K); }
+int fp6mi_prepack_native(int E, int Mb, void *native, const void *raw, size_t M, size_t K) { return fp6mi::prepack_native(E, Mb, native, raw, M, K); }
+int fp6mi_unpack_native(int E, int Mb, void *raw, const void *native, size_t M, size_t K) { return fp6mi::unpack_native(E, Mb, raw, native, M, K); }
+int fp6mi_relayout_ref_to_native(int E, int Mb, void *native, const void *ref, size_t M, size_t K)
+{
+    return fp6mi::relayout_ref_to_native(E, Mb, native, ref, M, K);
+}
+
+size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK) { return splitK > 1 ? (size_t)splitK * M * N * sizeof(float) : 0; }
+
+// Cost model, in microseconds, of the stream kernel on a part with `num_cus` compute units: workgroups run in rounds of
+// one per CU, a workgroup streams its weights at what one CU sustains, the whole chip cannot beat HBM, and a split
+// costs a second launch plus writing and re-reading the FP32 partial sums.
+int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus)
+{
+    if (M == 0 || N == 0 || K == 0 || num_cus <= 0) return 1;
+    const double cu_gbps = 60.0, hbm_gbps = 6000.0, launch_us = 3.0;
+    size_t       units = (K + 255) / 256, ntile = N <= 16 ? 16 : N <= 32 ? 32 : 64;
+    size_t       wgs = (M / 16 ? M / 16 : 1) * ((N + ntile - 1) / ntile);
+    double       best = 1e30;
+    int          best_s = 1;
+    for (int s = 1; s <= 64 && (size_t)s <= units; s++) {
+        double per_wg_bytes = (double)((units + s - 1) / s) * 3072.0;
+        double rounds = std::ceil((double)(wgs * (size_t)s) / (double)num_cus);
+        double t_cu = rounds * per_wg_bytes / (cu_gbps * 1e3);
+        double t_hbm = (double)wgs * (double)units * 3072.0 / (hbm_gbps * 1e3);
+        double t = launch_us + (t_cu > t_hbm ? t_cu : t_hbm);
+        if (s > 1) t += launch_us + 2.0 * (double)s * (double)M * (double)N * 4.0 / (hbm_gbps * 1e3);
+        if (t < best * 0.97) { best = t; best_s = s; }
+    }
+    return best_s;
+}
+
+static int check_gemm_args(int E, int Mb, const void *W, const void *sc, const void *B, const void *C, size_t M, size_t N, size_t K,
+                           const float *ws, int splitK)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (!W || !sc || !B || !C) return FP6MI_ERR_NULL;
+    if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
+    if (M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu || (N + 15) / 16 > 65535) return FP6MI_ERR_SHAPE;
+    if (splitK < 1 || splitK > 65535) return FP6MI_ERR_SPLITK;
+    if (splitK > 1 && !ws) return FP6MI_ERR_WORKSPACE;
+    if (!aligned16(W) || !aligned16(B) || !aligned16(C) || (ws && !aligned16(ws))) return FP6MI_ERR_ALIGN;
+    return FP6MI_OK;
+}
+
+int fp6mi_linear_native(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
+                        float *ws, int splitK)
+{
+    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK);
+}
+
+int fp6mi_relayout_ref_to_native_gpu(int E, int Mb, void *stream, void *native, const void *ref, size_t M, size_t K)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (!native || !ref) return FP6MI_ERR_NULL;
+    if (M == 0 || M % 64 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu || native == ref) return FP6MI_ERR_SHAPE;
+    if (!aligned16(native) || !aligned16(ref)) return FP6MI_ERR_ALIGN;
+    uint32_t units = (uint32_t)((K + 255) / 256);
+    size_t   blocks = (M / 16) * units;
+    dim3     grid((uint32_t)((blocks + 3) / 4));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (E == 3)
+        hipLaunchKernelGGL(relayout_ref_to_native<6>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native), static_cast<const uint8_t *>(ref),
+                           (uint32_t)M, (uint32_t)K, units);
+    else
+        hipLaunchKernelGGL(relayout_ref_to_native<5>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native), static_cast<const uint8_t *>(ref),
+                           (uint32_t)M, (uint32_t)K, units);
+    return (int)hipGetLastError();
+}
+
+int fp6mi_dequant_native_gpu(int E, int Mb, void *stream, void *out, const void *W, const void *sc, size_t M, size_t K)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (!out || !W || !sc) return FP6MI_ERR_NULL;
+    if (M == 0 || M % 16 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu) return FP6MI_ERR_SHAPE;
+    if (!aligned16(out) || !aligned16(W)) return FP6MI_ERR_ALIGN;
+    uint32_t units = (uint32_t)((K + 255) / 256);
+    size_t   blocks = (M / 16) * units;
+    dim3     grid((uint32_t)((blocks + 3) / 4));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (E == 3)
+        hipLaunchKernelGGL(dequant_native<6>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
+                           static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
+    else
+        hipLaunchKernelGGL(dequant_native<5>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
+                           static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
+    return (int)hipGetLastError();
+}
+
+} // extern "C"

@@ -1,0 +1,26 @@
+// Internal declarations shared by the host code and the kernel translation unit.
+#ifndef FP6MI_INTERNAL_H
+#define FP6MI_INTERNAL_H
+
+#include <cmath>
+#include <cstddef>
+#include <cstdint>
+
+#include "../../include/fp6mi.h"
+
+namespace fp6mi {
+
+inline bool supported(int E, int Mbits) { return Mbits == 2 && (E == 2 || E == 3); }
+
+// fp6mi_host.cpp
+int    prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K);
+int    unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K);
+int    dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16);
+size_t native_block_bytes(int x);
+size_t native_bytes(int E, int Mb, size_t M, size_t K);
+int    prepack_native(int E, int Mb, void *native, const void *raw, size_t M, size_t K);
+int    unpack_native(int E, int Mb, void *raw, const void *native, size_t M, size_t K);
+int    relayout_ref_to_native(int E, int Mb, void *native, const void *packed_ref, size_t M, size_t K);
+
+} // namespace fp6mi
+#endif

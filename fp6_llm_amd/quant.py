@@ -1,0 +1,85 @@
+"""FP16/FP32 -> FPx quantizer with per-row absmax scales, and raw-tensor packing.
+
+The reference ships only a truncating FP16->FP6 cast that is not wired into any API (fp6_llm/csrc/utils/weight_quant.h:9-105,
+"To be used in the future"); this one rounds to nearest, ties to even, clamps at the format maximum and covers e2m2 too.
+It is the step before the linear-layer path: it produces the raw int32 tensor that weight_prepacking*_cpu consumes.
+"""
+import numpy as np
+
+
+def _check(E, M):
+    if (E, M) not in ((3, 2), (2, 2)):
+        raise ValueError("unsupported format e%dm%d" % (E, M))
+    return 1 + E + M
+
+
+def magnitudes(E, M):
+    """Ascending non-negative values of the format; index == magnitude bits of the code (exponent all-ones is ordinary)."""
+    _check(E, M)
+    bias = (1 << (E - 1)) - 1
+    vals = []
+    for e in range(1 << E):
+        for m in range(1 << M):
+            vals.append(2.0 ** (1 - bias) * m / (1 << M) if e == 0 else 2.0 ** (e - bias) * (1 + m / (1 << M)))
+    return np.array(vals, dtype=np.float64)
+
+
+def max_value(E, M):
+    return float(magnitudes(E, M)[-1])
+
+
+def quantize_codes(values, E=3, M=2):
+    """values (any float array, already divided by the scale) -> uint8 codes, round-to-nearest, ties to the even code."""
+    x = _check(E, M)
+    v = np.asarray(values, dtype=np.float64)
+    mags = magnitudes(E, M)
+    a = np.minimum(np.abs(v), mags[-1])
+    hi = np.clip(np.searchsorted(mags, a, side="left"), 0, len(mags) - 1)   # first magnitude >= a
+    lo = np.maximum(hi - 1, 0)
+    d_hi, d_lo = mags[hi] - a, a - mags[lo]
+    pick_lo = (d_lo < d_hi) | ((d_lo == d_hi) & (lo % 2 == 0))
+    idx = np.where(pick_lo, lo, hi).astype(np.uint8)
+    sign = np.signbit(v).astype(np.uint8)
+    return (sign << (x - 1)) | idx
+
+
+def quantize_rowwise(weight, E=3, M=2):
+    """weight [OC, IC] float -> (codes uint8 [OC, IC], scales float16 [OC]) with scale = absmax(row) / max_value,
+    rounded to fp16 first so that codes are chosen against the scale that will actually be applied."""
+    w = np.asarray(weight, dtype=np.float64)
+    absmax = np.abs(w).max(axis=1)
+    scale = (absmax / max_value(E, M)).astype(np.float16)
+    scale = np.where(scale == 0, np.float16(1.0), scale).astype(np.float16)
+    return quantize_codes(w / scale.astype(np.float64)[:, None], E, M), scale
+
+
+def pack_raw(codes, E=3, M=2):
+    """codes uint8 [OC, IC] -> int32 [OC, IC/32*x]: each row an MSB-first bitstream carried in little-endian int32 words,
+    the raw weight format of the reference (fp6_llm/csrc/utils/common.h:4-19; worked example
+    tests/python/kernel_test_fpx.py:124-131)."""
+    x = _check(E, M)
+    c = np.asarray(codes, dtype=np.uint8)
+    if c.ndim != 2 or c.shape[1] % 32:
+        raise ValueError("codes must be [OC, IC] with IC % 32 == 0")
+    if (c >> x).any():
+        raise ValueError("a code does not fit in %d bits" % x)
+    shifts = np.arange(x - 1, -1, -1, dtype=np.uint8)
+    bits = (c[:, :, None] >> shifts) & 1
+    return np.packbits(bits.reshape(c.shape[0], -1), axis=1, bitorder="big").view(np.int32)
+
+
+def unpack_raw(raw, E=3, M=2):
+    """Inverse of pack_raw."""
+    x = _check(E, M)
+    b = np.ascontiguousarray(raw).view(np.uint8)
+    bits = np.unpackbits(b, axis=1, bitorder="big").reshape(b.shape[0], -1, x)
+    return (bits << np.arange(x - 1, -1, -1, dtype=np.uint8)).sum(axis=2).astype(np.uint8)
+
+
+def dequantize_codes(codes, scales, E=3, M=2):
+    """float64 value(code) * scale, for checks."""
+    x = _check(E, M)
+    c = np.asarray(codes)
+    mags = magnitudes(E, M)
+    v = np.where(c >> (x - 1), -1.0, 1.0) * mags[c & ((1 << (x - 1)) - 1)]
+    return v * np.asarray(scales, dtype=np.float64)[:, None]

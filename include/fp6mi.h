@@ -1,0 +1,93 @@
+/*
+ * fp6mi.h -- C ABI of the MI355X (gfx950) FPx x FP16 linear-layer engine.
+ *
+ * Plain C: pointers, sizes and ints only.  This is the boundary a host binding (ctypes, pybind, cgo, JNI ...)
+ * attaches to; the C++ header fp6_llm_amd/csrc/fp6_linear.h and the Python package fp6_llm_amd are thin layers
+ * over exactly these symbols.  Citations name the interface of usyd-fsalab/fp6_llm that each entry replaces
+ * (paths relative to that repository).
+ *
+ * Conventions (same as the reference, fp6_llm/csrc/fp6_linear.cu:149-159):
+ *   M = OC (weight rows), K = IC, N = batch.  Weights are x = 1+E+M bit codes, (E,M) in {(3,2), (2,2)}.
+ *   "raw" weights     : row-major [M,K] codes, per-row MSB-first bitstream, M*K*x/8 bytes.
+ *   "ref" layout      : the reference's prepacked layout (utils/weight_prepacking.h:118-196), same byte count.
+ *   "native" layout   : this engine's gfx950 layout, fp6mi_native_bytes() bytes (K padded to 256).
+ *   activations B     : fp16 [N,K] row-major;  output C : fp16 [N,M] row-major;  scales : fp16 [M].
+ *
+ * Return value of every int function: 0 on success, a negative FP6MI_ERR_* for rejected arguments, or a positive
+ * hipError_t from the runtime.  Nothing here aborts the process.  GPU entry points enqueue on `stream`
+ * (a hipStream_t passed as void*, NULL = the default stream) and do not synchronize.
+ */
+#ifndef FP6MI_H
+#define FP6MI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FP6MI_OK 0
+#define FP6MI_ERR_FORMAT (-1)    /* (E,M) is not (3,2) or (2,2)             */
+#define FP6MI_ERR_SHAPE (-2)     /* M % 256, K % 64, N > 0 or size overflow */
+#define FP6MI_ERR_NULL (-3)      /* a required pointer is NULL              */
+#define FP6MI_ERR_WORKSPACE (-4) /* splitK > 1 without a workspace          */
+#define FP6MI_ERR_SPLITK (-5)    /* splitK < 1                              */
+#define FP6MI_ERR_ALIGN (-6)     /* a device pointer is not 16-byte aligned */
+
+const char *fp6mi_error_string(int code);
+int         fp6mi_version(void);
+
+/* ------------------------------------------------------------------------------------------------ CPU side */
+
+/* Replaces weight_matrix_prepacking / weight_matrix_prepacking_fp_eXmY (fp6_llm/csrc/fp6_linear.cuh:36-37,
+ * utils/weight_prepacking.h:199-211): raw -> reference layout, bit-exact.  `packed` may alias `raw`.
+ * Requires M % 64 == 0 and K % 64 == 0 like the reference (utils/weight_prepacking.h:121-122). */
+int fp6mi_prepack_ref(int E, int Mbits, void *packed, const void *raw, size_t M, size_t K);
+
+/* Replaces DeQuantMatrix_FP6_To_FP16 / dequant_matrix_fp_eXmY_to_fp16 (fp6_llm/csrc/fp6_linear.cuh:42-43,
+ * utils/weight_dequant.h:10-61): raw -> fp16 [M,K], out = fp16_rn(value(code) * scale[row]), bit-exact. */
+int fp6mi_dequant(int E, int Mbits, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16);
+
+/* Inverse of fp6mi_prepack_ref (no counterpart in the reference): reference layout -> raw. */
+int fp6mi_unpack_ref(int E, int Mbits, void *raw, const void *packed, size_t M, size_t K);
+
+/* Native gfx950 layout (no counterpart in the reference; the reference's layout targets 32-lane warps and
+ * mma.m16n8k16 fragments, utils/weight_prepacking.h:39-85).  Requires M % 16 == 0, K % 64 == 0. */
+size_t fp6mi_native_bytes(int E, int Mbits, size_t M, size_t K);
+int    fp6mi_prepack_native(int E, int Mbits, void *native, const void *raw, size_t M, size_t K);
+int    fp6mi_relayout_ref_to_native(int E, int Mbits, void *native, const void *packed_ref, size_t M, size_t K);
+int    fp6mi_unpack_native(int E, int Mbits, void *raw, const void *native, size_t M, size_t K);
+
+/* Split-K choice for an MI355X-class part with `num_cus` compute units (replaces the role of
+ * HeuristicFuntion_SplitK, fp6_llm/__init__.py:13-23, whose model of one CTA per 512x64 outputs does not fit
+ * this kernel).  Returns a value in [1, 64]. */
+int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus);
+
+/* Bytes of the split-K workspace the GEMM entry points need: splitK*M*N floats (fp6_llm/csrc/fp6_linear.cuh:17),
+ * 0 when splitK == 1. */
+size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK);
+
+/* ------------------------------------------------------------------------------------------------ GPU side */
+
+/* The GEMM on native-layout weights: C[N,M] = B[N,K] . dequant(W)[M,K]^T, FP32 accumulation, fp16 output.
+ * Same argument meaning as fp_eXmY_linear_kernel (fp6_llm/csrc/fp6_linear.cuh:20-32) except that W is the
+ * native layout.  splitK > 1 splits K across workgroups; partial sums go to `workspace`
+ * ([splitK][N][M] floats, layout of include/kernel_matmul.cuh:183) and a reduction kernel
+ * (role of include/kernel_reduction.cuh:28-47) produces C.  M % 256 == 0, K % 64 == 0, N >= 1. */
+int fp6mi_linear_native(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
+                        const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK);
+
+/* Device-side conversion reference layout -> native layout (both device pointers), run once per weight matrix. */
+int fp6mi_relayout_ref_to_native_gpu(int E, int Mbits, void *stream, void *native_dev, const void *packed_ref_dev,
+                                     size_t M, size_t K);
+
+/* Device-side dequantisation of native-layout weights to fp16 [M,K]: the same arithmetic the GEMM applies in
+ * registers, made visible.  Bit-exact to fp6mi_dequant of the corresponding raw weights. */
+int fp6mi_dequant_native_gpu(int E, int Mbits, void *stream, void *out_f16_dev, const void *W_native_dev,
+                             const void *scales_f16_dev, size_t M, size_t K);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FP6MI_H */

@@ -1,0 +1,289 @@
+"""TEST INFRASTRUCTURE ONLY -- Python front end of the CPU oracle for the FPx linear-layer path.
+
+Only tests/, ``__graft_entry__.smoke()`` and ``bench.py``'s ``cpu_baseline`` leg may import this package, and
+only as the checker / timed CPU baseline.  The product (``fp6_llm_amd``) never imports it.
+
+Three layers live here:
+
+* ``liborc.so`` (``fpx_oracle.c``): scalar C restatement of the reference algorithm, reached through ctypes.
+* numpy closed forms that do NOT share code with the C restatement (``prepack_closed_form``, ``value_table``,
+  ``codes_to_raw``/``raw_to_codes``): used to cross-examine it.
+* ``ref_prepack``: the reference's own ``weight_prepacking.h`` compiled unmodified (``oracle/_ref``), when built.
+"""
+import ctypes
+import os
+import subprocess
+from fractions import Fraction
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+_REF = None
+
+
+def build(force=False):
+    """Compile liborc.so (and oracle/_ref when the reference checkout exists) with the Makefile beside this file."""
+    if force:
+        subprocess.run(["make", "-C", _HERE, "clean"], check=True, capture_output=True)
+    subprocess.run(["make", "-C", _HERE], check=True, capture_output=True)
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        path = os.path.join(_HERE, "liborc.so")
+        if not os.path.exists(path):
+            build()
+        L = ctypes.CDLL(path)
+        u8p, u16p, f32p = ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p
+        L.orc_prepack.argtypes = [ctypes.c_int, ctypes.c_int, u8p, u8p, ctypes.c_size_t, ctypes.c_size_t]
+        L.orc_prepack.restype = ctypes.c_int
+        L.orc_unpack_codes.argtypes = [ctypes.c_int, ctypes.c_int, u8p, u8p, ctypes.c_size_t, ctypes.c_size_t]
+        L.orc_unpack_codes.restype = ctypes.c_int
+        L.orc_dequant.argtypes = [ctypes.c_int, ctypes.c_int, u16p, u8p, ctypes.c_size_t, ctypes.c_size_t, u16p]
+        L.orc_dequant.restype = ctypes.c_int
+        L.orc_splitk_range.argtypes = [ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                       ctypes.POINTER(ctypes.c_size_t), ctypes.POINTER(ctypes.c_size_t)]
+        L.orc_splitk_range.restype = None
+        L.orc_splitk_reduce.argtypes = [u16p, f32p, ctypes.c_size_t, ctypes.c_int]
+        L.orc_splitk_reduce.restype = None
+        L.orc_gemm.argtypes = [u16p, u16p, u16p, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_size_t, ctypes.c_int]
+        L.orc_gemm.restype = ctypes.c_int
+        L.orc_tile_n.argtypes = [ctypes.c_size_t]
+        L.orc_tile_n.restype = ctypes.c_int
+        L.orc_num_wave.argtypes = [ctypes.c_long] * 4
+        L.orc_num_wave.restype = ctypes.c_double
+        L.orc_heuristic_splitk.argtypes = [ctypes.c_long] * 3
+        L.orc_heuristic_splitk.restype = ctypes.c_int
+        L.orc_float_to_half.argtypes = [ctypes.c_float]
+        L.orc_float_to_half.restype = ctypes.c_uint16
+        L.orc_half_to_float.argtypes = [ctypes.c_uint16]
+        L.orc_half_to_float.restype = ctypes.c_float
+        _LIB = L
+    return _LIB
+
+
+def ref_lib():
+    """The reference's own prepacker (oracle/_ref/libref_prepack.so) or None when it was never built."""
+    global _REF
+    if _REF is None:
+        path = os.path.join(_HERE, "_ref", "libref_prepack.so")
+        if not os.path.exists(path):
+            return None
+        R = ctypes.CDLL(path)
+        R.ref_weight_matrix_prepacking_fp_eXmY.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                           ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
+        R.ref_weight_matrix_prepacking_fp_eXmY.restype = None
+        R.ref_weight_matrix_prepacking.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
+        R.ref_weight_matrix_prepacking.restype = None
+        _REF = R
+    return _REF
+
+
+def _ptr(a):
+    return a.ctypes.data_as(ctypes.c_void_p)
+
+
+def bit_width(E, M):
+    return 1 + E + M
+
+
+def _as_bytes(raw):
+    """Accepts int32 [OC, IC/32*x] or uint8 [OC, IC*x/8]; returns a contiguous uint8 [OC, row_bytes] view."""
+    raw = np.ascontiguousarray(raw)
+    if raw.dtype != np.uint8:
+        raw = raw.view(np.uint8)
+    return raw
+
+
+# ---------------------------------------------------------------------------------------------- C restatement
+
+
+def prepack(raw, E=3, M=2):
+    """Restates weight_matrix_prepacking_x_bit (utils/weight_prepacking.h:118-196). Returns uint8 of raw's shape."""
+    b = _as_bytes(raw)
+    rows, row_bytes = b.shape
+    K = row_bytes * 8 // bit_width(E, M)
+    out = np.empty_like(b)
+    rc = lib().orc_prepack(E, M, _ptr(out), _ptr(b), rows, K)
+    if rc != 0:
+        raise ValueError("orc_prepack rejected E=%d M=%d rows=%d K=%d" % (E, M, rows, K))
+    return out
+
+
+def unpack_codes(raw, E=3, M=2):
+    b = _as_bytes(raw)
+    rows, row_bytes = b.shape
+    K = row_bytes * 8 // bit_width(E, M)
+    codes = np.empty((rows, K), dtype=np.uint8)
+    rc = lib().orc_unpack_codes(E, M, _ptr(codes), _ptr(b), rows, K)
+    if rc != 0:
+        raise ValueError("orc_unpack_codes rejected the input")
+    return codes
+
+
+def dequant(raw, scale, E=3, M=2):
+    """Restates DeQuantMatrix_FPx_To_FP16 (utils/weight_dequant.h:10-48). scale: float16 [OC]. Returns float16 [OC, IC]."""
+    b = _as_bytes(raw)
+    rows, row_bytes = b.shape
+    K = row_bytes * 8 // bit_width(E, M)
+    s = np.ascontiguousarray(scale, dtype=np.float16)
+    assert s.shape == (rows,)
+    out = np.empty((rows, K), dtype=np.float16)
+    rc = lib().orc_dequant(E, M, _ptr(out), _ptr(b), rows, K, _ptr(s))
+    if rc != 0:
+        raise ValueError("orc_dequant rejected the input")
+    return out
+
+
+def gemm(wdq, x, splitK=1):
+    """out[N, OC] = fp16_rn(sum_k float(wdq[m,k]) * float(x[n,k])), FP32 accumulation, reference split-K partition."""
+    wdq = np.ascontiguousarray(wdq, dtype=np.float16)
+    x = np.ascontiguousarray(x, dtype=np.float16)
+    Mg, K = wdq.shape
+    N = x.shape[0]
+    assert x.shape[1] == K
+    out = np.empty((N, Mg), dtype=np.float16)
+    rc = lib().orc_gemm(_ptr(out), _ptr(wdq), _ptr(x), Mg, N, K, splitK)
+    if rc != 0:
+        raise ValueError("orc_gemm rejected the input")
+    return out
+
+
+def splitk_range(K, splitK, split):
+    a, b = ctypes.c_size_t(), ctypes.c_size_t()
+    lib().orc_splitk_range(K, splitK, split, ctypes.byref(a), ctypes.byref(b))
+    return a.value, b.value
+
+
+def splitk_reduce(workspace):
+    """workspace float32 [splitK, N, OC] -> float16 [N, OC] (include/kernel_reduction.cuh:28-47)."""
+    ws = np.ascontiguousarray(workspace, dtype=np.float32)
+    s = ws.shape[0]
+    out = np.empty(ws.shape[1:], dtype=np.float16)
+    lib().orc_splitk_reduce(_ptr(out), _ptr(ws), out.size, s)
+    return out
+
+
+def tile_n(N):
+    return lib().orc_tile_n(N)
+
+
+def num_wave(M, N, splitK, sms):
+    return lib().orc_num_wave(M, N, splitK, sms)
+
+
+def heuristic_splitk(M, N, sms):
+    return lib().orc_heuristic_splitk(M, N, sms)
+
+
+# ---------------------------------------------------------------------------------------------- the real reference
+
+
+def ref_prepack(raw, E=3, M=2):
+    """The reference's own weight_matrix_prepacking_fp_eXmY. Input is padded: the reference reads one byte past it."""
+    R = ref_lib()
+    if R is None:
+        raise RuntimeError("oracle/_ref is not built (needs the reference checkout)")
+    b = _as_bytes(raw)
+    rows, row_bytes = b.shape
+    K = row_bytes * 8 // bit_width(E, M)
+    padded = np.zeros(b.size + 64, dtype=np.uint8)
+    padded[: b.size] = b.reshape(-1)
+    out = np.zeros(b.size + 64, dtype=np.uint8)
+    R.ref_weight_matrix_prepacking_fp_eXmY(E, M, _ptr(out), _ptr(padded), rows, K)
+    return out[: b.size].reshape(b.shape).copy()
+
+
+# ---------------------------------------------------------------------------------------------- independent numpy forms
+
+
+def codes_to_raw(codes, E=3, M=2):
+    """[OC, IC] codes -> uint8 [OC, IC*x/8]: per-row MSB-first bitstream (bit 0 = MSB of byte 0)."""
+    x = bit_width(E, M)
+    codes = np.asarray(codes, dtype=np.uint8)
+    bits = (codes[:, :, None] >> np.arange(x - 1, -1, -1, dtype=np.uint8)) & 1
+    return np.packbits(bits.reshape(codes.shape[0], -1), axis=1, bitorder="big")
+
+
+def raw_to_codes(raw, E=3, M=2):
+    x = bit_width(E, M)
+    b = _as_bytes(raw)
+    bits = np.unpackbits(b, axis=1, bitorder="big").reshape(b.shape[0], -1, x)
+    weights = (1 << np.arange(x - 1, -1, -1)).astype(np.uint8)
+    return (bits * weights).sum(axis=2).astype(np.uint8)
+
+
+def value_of_code(code, E=3, M=2):
+    """Format definition in exact arithmetic: (-1)^s 2^(e-b)(1+m/2^M), e=0 => (-1)^s 2^(1-b) m/2^M, b=2^(E-1)-1.
+    The all-ones exponent is an ordinary value (utils/weight_quant.h:22-25: FP6 max 28, min subnormal 0.0625)."""
+    x = bit_width(E, M)
+    s = (code >> (x - 1)) & 1
+    e = (code >> M) & ((1 << E) - 1)
+    m = code & ((1 << M) - 1)
+    b = (1 << (E - 1)) - 1
+    if e == 0:
+        v = Fraction(2) ** (1 - b) * Fraction(m, 1 << M)
+    else:
+        v = Fraction(2) ** (e - b) * (1 + Fraction(m, 1 << M))
+    return -v if s else v
+
+
+def value_table(E=3, M=2):
+    x = bit_width(E, M)
+    tab = np.array([float(value_of_code(c, E, M)) for c in range(1 << x)], dtype=np.float64)
+    sign = np.where(np.arange(1 << x) >> (x - 1), -1.0, 1.0)
+    return np.copysign(tab, sign)  # keeps the sign of the negative-zero code (sign bit set, all other bits clear)
+
+
+_ORDER = {
+    4: [2, 6, 4, 8, 1, 5, 3, 7],
+    2: [2, 6, 10, 14, 4, 8, 12, 16, 1, 5, 9, 13, 3, 7, 11, 15],
+    1: [2, 6, 10, 14, 18, 22, 26, 30, 4, 8, 12, 16, 20, 24, 28, 32,
+        1, 5, 9, 13, 17, 21, 25, 29, 3, 7, 11, 15, 19, 23, 27, 31],
+}
+
+
+def prepack_closed_form(codes, E=3, M=2):
+    """Reference layout from a closed-form index map (no passes, no per-lane streams): for every 32-bit word of a
+    segment array and every fragment position in it, the (row, column) whose bits sit there.
+    word = ((i*(K/16) + j)*w + q)*32 + lane; fragment p (MSB first) holds pre-interleave fragment order_w[p]-1 = pre;
+    pre -> 16-row block k = q*(4/w) + pre//8, element el = pre%8; lane = 4g+t;
+    row = 64i + 16k + g + 8*((el>>1)&1), col = 16j + 2t + (el&1) + 8*(el>>2)."""
+    x = bit_width(E, M)
+    codes = np.asarray(codes, dtype=np.uint32)
+    rows, K = codes.shape
+    out = []
+    consumed = 0
+    for w in (1, 2, 4):
+        if not (x & w):
+            continue
+        shift = x - consumed - w  # segments are cut MSB-down in the order 1,2,4
+        consumed += w
+        piece = (codes >> shift) & ((1 << w) - 1)
+        nfrag = 32 // w
+        i, j, q, lane, p = np.meshgrid(np.arange(rows // 64), np.arange(K // 16), np.arange(w), np.arange(32),
+                                       np.arange(nfrag), indexing="ij")
+        pre = np.array(_ORDER[w])[p] - 1
+        k = q * (4 // w) + pre // 8
+        el = pre % 8
+        g, t = lane // 4, lane % 4
+        row = 64 * i + 16 * k + g + 8 * ((el >> 1) & 1)
+        col = 16 * j + 2 * t + (el & 1) + 8 * (el >> 2)
+        frag = piece[row, col].astype(np.uint64) << (32 - w * (p + 1)).astype(np.uint64)
+        words = frag.sum(axis=-1).astype(np.uint32)  # fragments do not overlap, so the sum is an OR
+        out.append(words.reshape(-1).view(np.uint8))
+    return np.concatenate(out).reshape(rows, -1)
+
+
+def dequant_from_definition(codes, scale, E=3, M=2):
+    """fp16_rn(value(code) * scale) in float64 (the product has <= 3+11 significant bits, so it is exact)."""
+    tab = value_table(E, M)
+    prod = tab[np.asarray(codes)] * np.asarray(scale, dtype=np.float16).astype(np.float64)[:, None]
+    return prod.astype(np.float16)
+
+
+def gemm_f64(wdq, x):
+    """float64 accumulation of the dequantized weights: the arbiter for GEMM tolerance checks. Returns float64 [N, OC]."""
+    return np.asarray(x, dtype=np.float64) @ np.asarray(wdq, dtype=np.float64).T

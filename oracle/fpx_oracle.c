@@ -1,0 +1,320 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- CPU restatement of the FPx (FP6_e3m2 / FP5_e2m2) linear-layer path of
+ * usyd-fsalab/fp6_llm.  Nothing in the product links, loads or calls this file: only tests/,
+ * __graft_entry__.smoke() and bench.py's cpu_baseline leg may use it, and only as the checker or as the
+ * timed CPU baseline.
+ *
+ * Plain scalar C, written to follow the reference's algorithm step by step (citations are paths relative to
+ * the reference checkout, file:line).  It is deliberately slow and simple.
+ *
+ * What pins each function (see tests/test_oracle_*.py):
+ *   orc_prepack      : byte-for-byte against the reference's own weight_prepacking.h compiled unmodified
+ *                      (oracle/_ref), the all-ones known answers in tests/python/kernel_test_fpx.py:88-131,
+ *                      an independent closed-form index formula, and bijection / in-place invariants.
+ *   orc_dequant      : the reference's weight_dequant.h needs CUDA's <nv/target> which this image lacks, so it
+ *                      cannot be compiled here; pinned instead by the all-ones known answers (-> 1.0 everywhere),
+ *                      the format constants of utils/weight_quant.h:22-25 (max 28, min subnormal 0.0625), and an
+ *                      exhaustive check of every (code, fp16 scale sample) against the format definition evaluated in
+ *                      exact rational arithmetic and rounded by Python's own IEEE binary16 packer.
+ *   orc_splitk_*     : closed forms (partition covers [0,K/64) exactly once, first K/64 % s splits one longer).
+ *   orc_heuristic    : hand-computed known answers.
+ *   orc_gemm         : the mathematical definition (fp32 accumulation of dequantized weights); checked against
+ *                      float64 numpy matmul and closed-form special cases (all-ones => IC, one-hot activations).
+ *                      Bit-level parity with the reference CUDA kernel is unpinned: no reference test asserts it.
+ */
+#include <stdint.h>
+#include <stddef.h>
+#include <stdlib.h>
+#include <string.h>
+#include <math.h>
+
+/* ------------------------------------------------------------------ IEEE binary16 <-> binary32 (software) */
+static float orc_h2f(uint16_t h)
+{
+    uint32_t sign = (uint32_t)(h >> 15) << 31;
+    int      e    = (h >> 10) & 0x1f;
+    uint32_t man  = h & 0x3ffu;
+    uint32_t bits;
+    if (e == 0) {
+        if (man == 0) {
+            bits = sign;
+        } else { /* subnormal: value = man * 2^-24, exact in binary32 */
+            float v = (float)man * 5.9604644775390625e-08f;
+            memcpy(&bits, &v, 4);
+            bits |= sign;
+        }
+    } else if (e == 31) {
+        bits = sign | 0x7f800000u | (man << 13);
+    } else {
+        bits = sign | ((uint32_t)(e - 15 + 127) << 23) | (man << 13);
+    }
+    float f;
+    memcpy(&f, &bits, 4);
+    return f;
+}
+
+/* round-to-nearest-even, the behaviour of __float2half_rn (utils/weight_dequant.h:43) */
+static uint16_t orc_f2h(float f)
+{
+    uint32_t x;
+    memcpy(&x, &f, 4);
+    uint16_t sign = (uint16_t)((x >> 16) & 0x8000u);
+    uint32_t ax   = x & 0x7fffffffu;
+    if (ax >= 0x7f800000u) { /* inf / nan */
+        return (uint16_t)(sign | 0x7c00u | ((ax > 0x7f800000u) ? 0x200u : 0u));
+    }
+    if (ax >= 0x477ff000u) { /* >= 65520 rounds to inf */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (ax < 0x33000001u) { /* <= 2^-25 : rounds to zero (ties-to-even at exactly 2^-25) */
+        return sign;
+    }
+    int      e   = (int)(ax >> 23) - 127;
+    uint32_t man = (ax & 0x7fffffu) | 0x800000u; /* 24-bit significand */
+    int      shift;                              /* bits dropped from the 24-bit significand */
+    uint32_t base;
+    if (e < -14) { /* subnormal half: unit 2^-24 */
+        shift = 13 + (-14 - e);
+        base  = 0;
+    } else {
+        shift = 13;
+        base  = (uint32_t)(e + 15) << 10;
+        man  &= 0x7fffffu;
+    }
+    uint32_t q    = man >> shift;
+    uint32_t rem  = man & ((1u << shift) - 1u);
+    uint32_t half = 1u << (shift - 1);
+    if (rem > half || (rem == half && (q & 1u))) q++;
+    return (uint16_t)(sign | (base + q)); /* carry out of the mantissa bumps the exponent correctly */
+}
+
+uint16_t orc_float_to_half(float f) { return orc_f2h(f); }
+float    orc_half_to_float(uint16_t h) { return orc_h2f(h); }
+
+/* ------------------------------------------------------------------ raw bitstream (utils/common.h:4-19)
+ * A row is an MSB-first bitstream: code c occupies bits [c*x, (c+1)*x), bit 0 being the MSB of byte 0.
+ * Returns the code left-aligned in a byte (code << (8-x)), like Extract_X_Bits_To_A_Byte, but never reads
+ * past `nbytes` (the reference touches one extra byte whose bits are masked away).
+ */
+static uint8_t orc_left_aligned_code(const uint8_t *bytes, size_t nbytes, size_t bit, int x)
+{
+    size_t   byte = bit >> 3;
+    int      off  = (int)(bit & 7);
+    uint32_t w    = (uint32_t)bytes[byte] << 8;
+    if (byte + 1 < nbytes) w |= bytes[byte + 1];
+    w = (w << off) & 0xffffu;
+    uint8_t top = (uint8_t)(w >> 8);
+    return (uint8_t)(top & (uint8_t)(0xff00u >> x));
+}
+
+static int orc_supported(int E, int M) { return (M == 2) && (E == 2 || E == 3); }
+
+/* codes[r*K + c] = right-aligned x-bit code */
+int orc_unpack_codes(int E, int M, uint8_t *codes, const uint8_t *raw, size_t rows, size_t K)
+{
+    if (!orc_supported(E, M)) return -1;
+    int    x         = 1 + E + M;
+    size_t row_bytes = K * x / 8;
+    for (size_t r = 0; r < rows; r++)
+        for (size_t c = 0; c < K; c++)
+            codes[r * K + c] = (uint8_t)(orc_left_aligned_code(raw + r * row_bytes, row_bytes, c * x, x) >> (8 - x));
+    return 0;
+}
+
+/* ------------------------------------------------------------------ prepacking (utils/weight_prepacking.h) */
+
+/* weight_prepacking.h:23-35 : from 8 left-aligned codes cut `w` bits at `bit_offset`, pack MSB-first into w bytes */
+static void orc_cut_segment(uint8_t *seg, const uint8_t padded[8], int w, int bit_offset)
+{
+    for (int i = 0; i < w; i++) seg[i] = 0;
+    for (int i = 0; i < 8; i++) {
+        uint8_t piece = (uint8_t)((uint8_t)(padded[i] << bit_offset) & (uint8_t)(0xff00u >> w));
+        int     pos   = i * w;
+        seg[pos >> 3] |= (uint8_t)(piece >> (pos & 7));
+    }
+}
+
+/* weight_prepacking.h:87-116 : per 32-bit word, output fragment p (MSB first) = input fragment order[p]-1 */
+static uint32_t orc_bit_interleave(uint32_t in, int w)
+{
+    static const int order1[32] = { 2, 6, 10, 14, 18, 22, 26, 30, 4, 8, 12, 16, 20, 24, 28, 32,
+                                    1, 5, 9, 13, 17, 21, 25, 29, 3, 7, 11, 15, 19, 23, 27, 31 };
+    static const int order2[16] = { 2, 6, 10, 14, 4, 8, 12, 16, 1, 5, 9, 13, 3, 7, 11, 15 };
+    static const int order4[8]  = { 2, 6, 4, 8, 1, 5, 3, 7 };
+    const int *order = (w == 1) ? order1 : (w == 2) ? order2 : order4;
+    uint32_t   top   = (w == 1) ? 0x80000000u : (w == 2) ? 0xc0000000u : 0xf0000000u;
+    uint32_t   out   = 0;
+    for (int p = 0; p < 32 / w; p++) {
+        uint32_t frag = (in << (w * (order[p] - 1))) & top;
+        out |= frag >> (p * w);
+    }
+    return out;
+}
+
+/*
+ * weight_prepacking.h:118-196.  `out` may alias `in` (the reference is used in place at
+ * tests/cpp/kernel_test_fp6.cu:27) because pass 1 buffers everything first.
+ * Returns 0, or -1 for unsupported (E,M) / shapes (the reference asserts M%64, K%64 at :121-122 and exits on
+ * unsupported formats at :209-210).
+ */
+int orc_prepack(int E, int M, uint8_t *out, const uint8_t *in, size_t rows, size_t K)
+{
+    if (!orc_supported(E, M) || rows % 64 || K % 64) return -1;
+    int    x         = 1 + E + M;
+    size_t row_bytes = K * x / 8;
+    int    widths[3] = { 1, 2, 4 };
+    /* per-lane byte streams for every segment that the bit width uses (pass 1 target) */
+    uint8_t *stream[3][32];
+    size_t   fill[3][32];
+    size_t   per_lane[3];
+    for (int s = 0; s < 3; s++) {
+        per_lane[s] = (x & widths[s]) ? rows * K * widths[s] / 8 / 32 : 0;
+        for (int t = 0; t < 32; t++) {
+            stream[s][t] = per_lane[s] ? (uint8_t *)malloc(per_lane[s]) : NULL;
+            fill[s][t]   = 0;
+        }
+    }
+    /* bit offsets at which the 1-, 2- and 4-bit pieces start inside a left-aligned code (:64-66) */
+    int offs[3] = { 0, x & 1, x & 3 };
+
+    /* pass 1 (:141-157): 64-row tile i, 16-column slice j, 16-row block k, row-in-octet l */
+    for (size_t i = 0; i < rows / 64; i++)
+        for (size_t j = 0; j < K / 16; j++)
+            for (size_t k = 0; k < 4; k++) {
+                size_t row0 = i * 64 + k * 16, col0 = j * 16;
+                for (int l = 0; l < 8; l++) {
+                    /* the four 1x8 strips of the 16x16 block that feed lanes 4l..4l+3 (:146-153):
+                       strip 0 = (row l, cols 0-7), 1 = (row l+8, cols 0-7), 2 = (row l, cols 8-15), 3 = (row l+8, cols 8-15) */
+                    const uint8_t *strip_row[4] = { in + (row0 + l) * row_bytes, in + (row0 + l + 8) * row_bytes,
+                                                    in + (row0 + l) * row_bytes, in + (row0 + l + 8) * row_bytes };
+                    size_t strip_col[4] = { col0, col0, col0 + 8, col0 + 8 };
+                    for (int t = 0; t < 4; t++) {
+                        uint8_t padded[8];
+                        for (int e = 0; e < 8; e++) { /* element e of lane t: strip e/2, strip column 2t + e%2 (:51-57) */
+                            int    sp  = e / 2;
+                            size_t col = strip_col[sp] + (size_t)(2 * t + (e & 1));
+                            padded[e]  = orc_left_aligned_code(strip_row[sp], row_bytes, col * x, x);
+                        }
+                        for (int s = 0; s < 3; s++) {
+                            if (!per_lane[s]) continue;
+                            uint8_t seg[4];
+                            orc_cut_segment(seg, padded, widths[s], offs[s]);
+                            for (int b = 0; b < widths[s]; b++) stream[s][4 * l + t][fill[s][4 * l + t]++] = seg[b];
+                        }
+                    }
+                }
+            }
+    /* passes 2 and 3 (:171-195): lane-interleave into 128-byte chunks with the bytes of each 32-bit word reversed,
+       then bit-interleave every 32-bit word.  Segment arrays follow each other in the order 1,2,4 (:131-133). */
+    uint8_t *dst = out;
+    for (int s = 0; s < 3; s++) {
+        if (!per_lane[s]) continue;
+        for (size_t c = 0; c < per_lane[s] / 4; c++)
+            for (int t = 0; t < 32; t++) {
+                const uint8_t *b4   = stream[s][t] + 4 * c;
+                uint32_t       word = ((uint32_t)b4[0] << 24) | ((uint32_t)b4[1] << 16) | ((uint32_t)b4[2] << 8) | b4[3];
+                word                = orc_bit_interleave(word, widths[s]);
+                uint8_t *o          = dst + c * 128 + (size_t)t * 4;
+                o[0] = (uint8_t)word; o[1] = (uint8_t)(word >> 8); o[2] = (uint8_t)(word >> 16); o[3] = (uint8_t)(word >> 24);
+            }
+        dst += per_lane[s] * 32;
+    }
+    for (int s = 0; s < 3; s++)
+        for (int t = 0; t < 32; t++) free(stream[s][t]);
+    return 0;
+}
+
+/* ------------------------------------------------------------------ dequantisation (utils/weight_dequant.h:10-48)
+ * fp16 bit pattern = sign<<15 | (magnitude bits of the code) << 8   (:30-40; RIGHT_SHIFT = 5-E puts the exponent
+ * field in the low bits of the fp16 exponent), times 2^(16-2^(E-1)) (:34-35), times float(scale[row]) in FP32,
+ * one round-to-nearest-even to fp16 (:43).  Input is the RAW (not prepacked) tensor.
+ */
+int orc_dequant(int E, int M, uint16_t *out, const uint8_t *raw, size_t rows, size_t K, const uint16_t *scale)
+{
+    if (!orc_supported(E, M) || K % 8) return -1;
+    int    x         = 1 + E + M;
+    size_t row_bytes = K * x / 8;
+    float  bias      = (float)(1u << (16 - (1 << (E - 1))));
+    for (size_t r = 0; r < rows; r++) {
+        float s = orc_h2f(scale[r]);
+        for (size_t c = 0; c < K; c++) {
+            uint8_t  la   = orc_left_aligned_code(raw + r * row_bytes, row_bytes, c * x, x); /* s eee mm 00 or s ee mm 000 */
+            uint32_t w    = (uint32_t)la << 24;
+            uint32_t mask = (0xffffffffu << (31 - (E + M))) & 0x7fffffffu; /* magnitude bits of the left-aligned code */
+            uint32_t h    = (w & 0x80000000u) | ((w & mask) >> (5 - E));
+            uint16_t hb   = (uint16_t)(h >> 16);
+            out[r * K + c] = orc_f2h(orc_h2f(hb) * bias * s);
+        }
+    }
+    return 0;
+}
+
+/* ------------------------------------------------------------------ split-K (include/kernel_matmul.cuh:54-70) */
+void orc_splitk_range(size_t K, int splitK, int split, size_t *first_block, size_t *num_blocks)
+{
+    size_t nb = K / 64, avg = nb / (size_t)splitK, extra = nb - avg * (size_t)splitK;
+    size_t start = avg * (size_t)split, n = avg;
+    if ((size_t)split < extra) { n++; start += (size_t)split; } else start += extra;
+    *first_block = start;
+    *num_blocks  = n;
+}
+
+/* include/kernel_reduction.cuh:28-47 : sequential FP32 sum over splits in index order, then RN to half */
+void orc_splitk_reduce(uint16_t *C, const float *workspace, size_t MN, int splitK)
+{
+    for (size_t i = 0; i < MN; i++) {
+        float acc = 0.0f;
+        for (int s = 0; s < splitK; s++) acc += workspace[(size_t)s * MN + i];
+        C[i] = orc_f2h(acc);
+    }
+}
+
+/* ------------------------------------------------------------------ GEMM definition
+ * out[n*M + m] = fp16_rn( sum_k float(Wdq[m*K+k]) * float(X[n*K+k]) ), FP32 accumulation in k order
+ * (include/ptx_mma.cuh:59-71 accumulates FP32; include/kernel_matmul.cuh:188 rounds once).  With splitK > 1 the
+ * partial sums follow orc_splitk_range and are combined by orc_splitk_reduce, like fp6_linear.cu:83-100.
+ */
+int orc_gemm(uint16_t *out, const uint16_t *Wdq, const uint16_t *X, size_t M, size_t N, size_t K, int splitK)
+{
+    if (splitK < 1 || K % 64) return -1;
+    float *ws = (float *)calloc((size_t)splitK * M * N, sizeof(float));
+    if (!ws) return -2;
+    for (int s = 0; s < splitK; s++) {
+        size_t b0, nb;
+        orc_splitk_range(K, splitK, s, &b0, &nb);
+        for (size_t n = 0; n < N; n++)
+            for (size_t m = 0; m < M; m++) {
+                float acc = 0.0f;
+                for (size_t k = b0 * 64; k < (b0 + nb) * 64; k++) acc += orc_h2f(Wdq[m * K + k]) * orc_h2f(X[n * K + k]);
+                ws[((size_t)s * N + n) * M + m] = acc;
+            }
+    }
+    orc_splitk_reduce(out, ws, M * N, splitK);
+    free(ws);
+    return 0;
+}
+
+/* ------------------------------------------------------------------ launcher logic */
+
+/* fp6_linear.cu:61-75 : batch bucket -> TILE_N of the CUDA kernel (8,16,32,64; everything above uses 64) */
+int orc_tile_n(size_t N)
+{
+    if (N <= 8) return 8;
+    if (N <= 16) return 16;
+    if (N <= 32) return 32;
+    return 64;
+}
+
+/* fp6_llm/__init__.py:6-23 */
+double orc_num_wave(long M, long N, long splitK, long sms)
+{
+    return ceil((double)M / 512.0) * ceil((double)N / 64.0) * (double)splitK / (double)sms;
+}
+int orc_heuristic_splitk(long M, long N, long sms)
+{
+    for (int i = 1; i < 100; i++) {
+        double w = orc_num_wave(M, N, i, sms);
+        if (w / ceil(w) >= 0.8) return i;
+    }
+    return 1;
+}
