@@ -87,7 +87,7 @@ def weight_prepacking_eXmY_cpu(EXPONENT, MANTISSA, fpx_tensor):
     """int32 CPU [OC, IC/32*x] raw codes -> same shape/dtype, the reference's prepacked layout, bit-exact."""
     OC, IC = _weight_shape(fpx_tensor, EXPONENT, MANTISSA, "fpx_tensor")
     if OC % 256 != 0 or IC % 64 != 0:
-        raise ValueError("weight_prepacking: need OC % 256 == 0 and IC % 64 == 0, got OC=%d IC=%d" % (OC, IC))
+        raise ValueError("weight_prepacking: need OC %% 256 == 0 and IC %% 64 == 0, got OC=%d IC=%d" % (OC, IC))
     src = _cpu_contig(fpx_tensor, "fpx_tensor")
     out = torch.empty_like(src)
     _lib.check(_lib.lib().fp6mi_prepack_ref(EXPONENT, MANTISSA, out.data_ptr(), src.data_ptr(), OC, IC), "fp6mi_prepack_ref")
@@ -201,7 +201,7 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
         raise ValueError("scales must be float16 [OC]")
     B, IC = in_feats.shape
     if OC % 256 != 0 or IC % 64 != 0 or B < 1:
-        raise ValueError("need OC % 256 == 0, IC % 64 == 0, B >= 1 (got OC=%d IC=%d B=%d)" % (OC, IC, B))
+        raise ValueError("need OC %% 256 == 0, IC %% 64 == 0, B >= 1 (got OC=%d IC=%d B=%d)" % (OC, IC, B))
     if native_weight.numel() * native_weight.element_size() != native_bytes(EXPONENT, MANTISSA, OC, IC):
         raise ValueError("native_weight has the wrong size for OC=%d IC=%d" % (OC, IC))
     if int(splitK) < 1:

@@ -99,32 +99,79 @@ __device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
 
 // ---------------------------------------------------------------------------------------------------------------
 // gemm_stream: weight-bandwidth-bound GEMM for small batches.
-//   grid  = (M/16 row tiles, splitK, ceil(N / (16*NT)))      block = WAVES wavefronts
-// A workgroup owns 16 output rows and 16*NT batch columns over the K blocks of its split; its wavefronts take the
+//   grid  = (M/(16*RT) row groups, splitK, ceil(N / (16*NT)))      block = WAVES wavefronts
+// A workgroup owns 16*RT output rows and 16*NT batch columns over the K blocks of its split; its wavefronts take the
 // blocks round-robin (K is split inside the workgroup), each streaming its weights HBM -> VGPR and its slice of the
-// activations L2 -> VGPR directly in MFMA B-operand order; partial accumulators are summed through LDS.
+// activations L2 -> VGPR directly in MFMA B-operand order (reused for the RT row tiles); the partial accumulators are
+// summed through LDS.  With PF the loads of the next K block are issued before the current one is consumed.
 // ---------------------------------------------------------------------------------------------------------------
-template <int XB, int NT, int WAVES>
+template <int XB, int NT, int RT> struct Stage {
+    WFrag<XB> w[RT];
+    v8h       x[8][NT];
+};
+
+template <int XB, int NT, int RT>
+__device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
+                                           const half_t *const (&xrow)[NT], const bool (&xok)[NT], int q, uint32_t K)
+{
+#pragma unroll
+    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
+#ifndef FP6MI_EXP_NOX
+#pragma unroll
+    for (int s = 0; s < 8; s++) {
+        uint32_t k = u * 256 + 32 * s;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            v8h z = { 0, 0, 0, 0, 0, 0, 0, 0 };
+            st.x[s][t] = (xok[t] && k + 8 * q < K) ? *reinterpret_cast<const v8h *>(xrow[t] + k) : z;
+        }
+    }
+#else
+#pragma unroll
+    for (int s = 0; s < 8; s++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) { v8h o = { 1, 1, 1, 1, 1, 1, 1, 1 }; st.x[s][t] = o; }
+#endif
+}
+
+template <int XB, int NT, int RT>
+__device__ __forceinline__ void consume_stage(const Stage<XB, NT, RT> &st, v4f (&acc)[RT][NT])
+{
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+        AOps<XB> a;
+        convert(st.w[r], a);
+#pragma unroll
+        for (int s = 0; s < 8; s++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.s[s], st.x[s][t], acc[r][t], 0, 0, 0);
+    }
+}
+
+template <int XB, int NT, int RT, int WAVES, bool PF>
 __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
                                                             const half_t *__restrict__ X, half_t *__restrict__ C,
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
                                                             uint32_t units, uint32_t splitK)
 {
-    __shared__ float red[WAVES][NT][256];
+    __shared__ float red[WAVES][RT * NT][256];
 
     const int      lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const int      col = lane & 15, q = lane >> 4;
-    const uint32_t R = blockIdx.x, split = blockIdx.y, nbase = blockIdx.z * (16 * NT);
+    const uint32_t R0 = blockIdx.x * RT, split = blockIdx.y, nbase = blockIdx.z * (16 * NT);
 
     const uint32_t avg = units / splitK, extra = units % splitK;
     const uint32_t u0 = split * avg + (split < extra ? split : extra);
     const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
 
-    const uint8_t *wrow = W + (size_t)R * units * Fmt<XB>::block_bytes;
+    const size_t   tile_stride = (size_t)units * Fmt<XB>::block_bytes;
+    const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
 
-    v4f acc[NT];
+    v4f acc[RT][NT];
 #pragma unroll
-    for (int t = 0; t < NT; t++) acc[t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
 
     const half_t *xrow[NT];
     bool          xok[NT];
@@ -135,38 +182,47 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         xrow[t]    = X + (size_t)(xok[t] ? n : 0) * K + 8 * q;
     }
 
-    for (uint32_t u = u0 + wave; u < u1; u += WAVES) {
-        WFrag<XB> wf = load_wfrag<XB>(wrow + (size_t)u * Fmt<XB>::block_bytes, lane);
-        v8h       xb[8][NT];
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            uint32_t k = u * 256 + 32 * s;
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                v8h z = { 0, 0, 0, 0, 0, 0, 0, 0 };
-                xb[s][t] = (xok[t] && k + 8 * q < K) ? *reinterpret_cast<const v8h *>(xrow[t] + k) : z;
+    // workgroups that share an L2 (ids congruent mod 8) start on different K blocks, so that the chip does not ask
+    // the same activation lines of the same L2 channel at the same moment
+    uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES);
+    if (PF) {
+        if (u < u1) {
+            Stage<XB, NT, RT> cur;
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, xok, q, K);
+            for (;;) {
+                uint32_t   un = u + WAVES;
+                const bool more = un < u1;
+                Stage<XB, NT, RT> nxt;
+                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, xok, q, K);
+                consume_stage<XB, NT, RT>(cur, acc);
+                if (!more) break;
+                cur = nxt;
+                u   = un;
             }
         }
-        AOps<XB> a;
-        convert(wf, a);
-#pragma unroll
-        for (int s = 0; s < 8; s++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) acc[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.s[s], xb[s][t], acc[t], 0, 0, 0);
+    } else {
+        for (; u < u1; u += WAVES) {
+            Stage<XB, NT, RT> cur;
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, xok, q, K);
+            consume_stage<XB, NT, RT>(cur, acc);
+        }
     }
 
-    // acc[t][i] = sum for output row 4q+i, batch column 16t+col
+    // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
 #pragma unroll
-    for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[wave][t][lane * 4]) = acc[t];
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[wave][r * NT + t][lane * 4]) = acc[r][t];
     __syncthreads();
 
-    for (int e = threadIdx.x; e < NT * 256; e += WAVES * kWave) {
-        int   t = e >> 8, r = e & 255, n = r >> 4, mm = r & 15;
+    for (int e = threadIdx.x; e < RT * NT * 256; e += WAVES * kWave) {
+        int   rt = e >> 8, i8 = e & 255, n = i8 >> 4, mm = i8 & 15;
+        int   r = rt / NT, t = rt % NT;
         int   idx = (((mm >> 2) * 16 + n) << 2) | (mm & 3);
         float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) sum += red[w][t][idx];
-        uint32_t ng = nbase + 16 * t + n, mg = R * 16 + mm;
+        for (int w = 0; w < WAVES; w++) sum += red[w][rt][idx];
+        uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
         if (ng < N) {
             float v = sum * ((float)scales[mg] * Fmt<XB>::post_scale);
             if (splitK == 1)
@@ -304,36 +360,62 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int XB, int NT, int WAVES>
+template <int XB, int NT, int RT, int WAVES, bool PF>
 int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
                   int splitK)
 {
     uint32_t units = (uint32_t)((K + 255) / 256);
-    dim3     grid((uint32_t)(M / 16), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    hipLaunchKernelGGL((gemm_stream<XB, NT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
+    dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
+    hipLaunchKernelGGL((gemm_stream<XB, NT, RT, WAVES, PF>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
                        static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M,
                        (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
     return (int)hipGetLastError();
 }
 
+struct StreamCfg { int nt, rt, waves; };
+
+// Launch shape of the stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M
+// as long as M/(16*rt) workgroups still cover the compute units; wavefronts per workgroup follow the K blocks available
+// to one split and the register budget (16 wavefronts leave 128 VGPRs each).
+inline StreamCfg pick_cfg(size_t M, size_t N, size_t K, int splitK, int cus)
+{
+    StreamCfg c;
+    c.nt = N <= 16 ? 1 : N <= 32 ? 2 : 4;
+    size_t tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
+    size_t nblk = (N + 16 * c.nt - 1) / (16 * c.nt);
+    c.rt = 1;
+    int max_rt = c.nt == 1 ? 4 : 2;
+    while (c.rt < max_rt && tiles % (2 * c.rt) == 0 && (tiles / (2 * c.rt)) * splitK * nblk >= (size_t)cus) c.rt *= 2;
+    int max_waves = (c.nt == 1 && c.rt <= 2) ? 16 : 8;
+    c.waves = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
+    if (c.waves > max_waves) c.waves = max_waves;
+    return c;
+}
+
+template <int XB>
+int launch_cfg(const StreamCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
+               size_t K, int splitK)
+{
+#define FP6MI_CASE(NT, RT, WV) \
+    if (c.nt == NT && c.rt == RT && c.waves == WV) return launch_stream<XB, NT, RT, WV, false>(st, W, sc, B, C, ws, M, N, K, splitK);
+    FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
+    FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
+    FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
+    FP6MI_CASE(2, 1, 4) FP6MI_CASE(2, 1, 8)
+    FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
+    FP6MI_CASE(4, 1, 4) FP6MI_CASE(4, 1, 8)
+    FP6MI_CASE(4, 2, 4) FP6MI_CASE(4, 2, 8)
+#undef FP6MI_CASE
+    return FP6MI_ERR_SHAPE;
+}
+
 template <int XB>
 int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
-                  int splitK)
+                  int splitK, const StreamCfg *forced)
 {
-    size_t units = (K + 255) / 256;
-    size_t per_split = (units + (size_t)splitK - 1) / (size_t)splitK;
-    int    rc;
-    if (N <= 16) {
-        if (per_split > 8) rc = launch_stream<XB, 1, 16>(st, W, sc, B, C, ws, M, N, K, splitK);
-        else if (per_split > 4) rc = launch_stream<XB, 1, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
-        else rc = launch_stream<XB, 1, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
-    } else if (N <= 32) {
-        if (per_split > 4) rc = launch_stream<XB, 2, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
-        else rc = launch_stream<XB, 2, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
-    } else {
-        if (per_split > 4) rc = launch_stream<XB, 4, 8>(st, W, sc, B, C, ws, M, N, K, splitK);
-        else rc = launch_stream<XB, 4, 4>(st, W, sc, B, C, ws, M, N, K, splitK);
-    }
+    StreamCfg c = forced ? *forced : pick_cfg(M, N, K, splitK, 256);
+    if ((M / 16) % c.rt) return FP6MI_ERR_SHAPE;
+    int rc = launch_cfg<XB>(c, st, W, sc, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
     if (splitK > 1) {
         size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
@@ -421,7 +503,17 @@ int fp6mi_linear_native(int E, int Mb, void *stream, const void *W, const void *
     int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
     if (rc != FP6MI_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK);
+    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr);
+}
+
+int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
+                            float *ws, int splitK, int n_tiles, int row_tiles, int waves)
+{
+    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    StreamCfg   c = { n_tiles, row_tiles, waves };
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, &c) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, &c);
 }
 
 int fp6mi_relayout_ref_to_native_gpu(int E, int Mb, void *stream, void *native, const void *ref, size_t M, size_t K)

@@ -63,9 +63,21 @@ def pack_raw(codes, E=3, M=2):
         raise ValueError("codes must be [OC, IC] with IC % 32 == 0")
     if (c >> x).any():
         raise ValueError("a code does not fit in %d bits" % x)
-    shifts = np.arange(x - 1, -1, -1, dtype=np.uint8)
-    bits = (c[:, :, None] >> shifts) & 1
-    return np.packbits(bits.reshape(c.shape[0], -1), axis=1, bitorder="big").view(np.int32)
+    if x == 6:   # 4 codes -> 3 bytes
+        q = c.reshape(c.shape[0], -1, 4)
+        out = np.empty((c.shape[0], q.shape[1], 3), dtype=np.uint8)
+        out[:, :, 0] = (q[:, :, 0] << 2) | (q[:, :, 1] >> 4)
+        out[:, :, 1] = (q[:, :, 1] << 4) | (q[:, :, 2] >> 2)
+        out[:, :, 2] = (q[:, :, 2] << 6) | q[:, :, 3]
+    else:        # 8 codes -> 5 bytes
+        q = c.reshape(c.shape[0], -1, 8)
+        out = np.empty((c.shape[0], q.shape[1], 5), dtype=np.uint8)
+        out[:, :, 0] = (q[:, :, 0] << 3) | (q[:, :, 1] >> 2)
+        out[:, :, 1] = (q[:, :, 1] << 6) | (q[:, :, 2] << 1) | (q[:, :, 3] >> 4)
+        out[:, :, 2] = (q[:, :, 3] << 4) | (q[:, :, 4] >> 1)
+        out[:, :, 3] = (q[:, :, 4] << 7) | (q[:, :, 5] << 2) | (q[:, :, 6] >> 3)
+        out[:, :, 4] = (q[:, :, 6] << 5) | q[:, :, 7]
+    return out.reshape(c.shape[0], -1).view(np.int32)
 
 
 def unpack_raw(raw, E=3, M=2):

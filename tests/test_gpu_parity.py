@@ -1,0 +1,274 @@
+"""GPU parity: the HIP path, called through the C ABI (ctypes) and through the reference-named Python API, against the
+CPU oracle on the same seeded inputs.
+
+Bars: bit-exact for prepack/relayout/dequant; for GEMM outputs
+    max_i |y_i - r_i| / max(|r_i|, rms(r)) <= 1e-2      (r = float64 accumulation of the oracle-dequantized weights)
+and the reference's own printed metric mean|err|/mean|ref| (tests/python/kernel_test_fp6.py:71-75) <= 2e-3.
+"""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import fp6_llm_amd as fp6
+from fp6_llm_amd import _lib, quant, synth
+
+pytestmark = pytest.mark.gpu
+
+FORMATS = [(3, 2), (2, 2)]
+TOL_MAX_REL = 1e-2
+TOL_MEAN_REL = 2e-3
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module", autouse=True)
+def _require_gpu_and_native_code():
+    assert torch.cuda.is_available(), "these tests need the MI355X"
+    assert "gfx950" in torch.cuda.get_device_properties(0).gcnArchName
+    _lib.lib()  # raises if libfp6mi.so is missing: there is no fallback to test
+
+
+def rel_errors(y, ref):
+    y = np.asarray(y, dtype=np.float64)
+    ref = np.asarray(ref, dtype=np.float64)
+    den = np.maximum(np.abs(ref), np.sqrt((ref ** 2).mean()))
+    return float((np.abs(y - ref) / den).max()), float(np.abs(y - ref).mean() / np.abs(ref).mean())
+
+
+def check_close(y, ref, what):
+    mx, mean = rel_errors(y, ref)
+    assert mx <= TOL_MAX_REL and mean <= TOL_MEAN_REL, "%s: max rel %.3e mean rel %.3e" % (what, mx, mean)
+
+
+def gemm_capi(E, M, native_dev, scales_dev, x_dev, OC, splitK=1, cfg=None):
+    """One GEMM through the C ABI with explicitly managed buffers."""
+    L = _lib.lib()
+    B, IC = x_dev.shape
+    out = torch.full((B, OC), float("nan"), dtype=torch.float16, device=DEV)
+    ws = torch.empty(max(1, splitK * B * OC), dtype=torch.float32, device=DEV) if splitK > 1 else None
+    stream = torch.cuda.current_stream().cuda_stream
+    args = [E, M, stream, native_dev.data_ptr(), scales_dev.data_ptr(), x_dev.data_ptr(), out.data_ptr(), OC, B, IC,
+            ws.data_ptr() if ws is not None else None, splitK]
+    rc = L.fp6mi_linear_native(*args) if cfg is None else L.fp6mi_linear_native_cfg(*args, *cfg)
+    assert rc == 0, L.fp6mi_error_string(rc)
+    torch.cuda.synchronize()
+    return out.cpu().numpy()
+
+
+def upload(raw, sc, x, E, M):
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    return native, torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+
+
+# ------------------------------------------------------------------------------------------------ bit-exact parts
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("OC,IC", [(256, 64), (256, 320), (512, 1024), (1024, 4096)])
+def test_relayout_and_dequant_bit_exact(E, M, OC, IC):
+    print("case relayout/dequant", E, M, OC, IC, flush=True)
+    raw, sc, _ = synth.uniform_problem(OC * 7 + IC, OC, IC, 1, E, M)
+    t = torch.from_numpy(raw)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, t)
+    assert packed.numpy().tobytes() == oracle.prepack(raw, E, M).tobytes()
+    native_cpu = fp6.weight_prepacking_native_cpu(E, M, t)
+    native_gpu = fp6.to_native(packed.to(DEV), E, M)
+    torch.cuda.synchronize()
+    assert torch.equal(native_gpu.cpu(), native_cpu)
+    dq = fp6.weight_dequant_native_cuda(E, M, native_gpu, torch.from_numpy(sc).to(DEV), OC, IC).cpu().numpy()
+    assert (dq.view(np.uint16) == oracle.dequant(raw, sc, E, M).view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_gpu_dequant_every_code_with_awkward_scales(E, M):
+    """All codes (incl. negative zero and subnormal inputs) times scales that make subnormal / overflowing products."""
+    x = 1 + E + M
+    OC, IC = 256, 64
+    codes = np.resize(np.arange(1 << x, dtype=np.uint8), (OC, IC))
+    raw = quant.pack_raw(codes, E, M)
+    bits = np.concatenate([np.arange(1, 0x7C00, 0x7C00 // 250)[:250], [0, 0x0001, 0x03FF, 0x0400, 0x7BFF, 0x8400]]).astype(np.uint16)
+    sc = bits[:OC].view(np.float16).copy()
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    dq = fp6.weight_dequant_native_cuda(E, M, native, torch.from_numpy(sc).to(DEV), OC, IC).cpu().numpy()
+    assert (dq.view(np.uint16) == oracle.dequant(raw, sc, E, M).view(np.uint16)).all()
+
+
+# ------------------------------------------------------------------------------------------------ GEMM vs oracle
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_config1_cpu_reference_case(E, M):
+    """OC=256, IC=1024, BS=1: the reference's CPU-runnable case, checked against the scalar C oracle end to end."""
+    print("case config1", E, M, flush=True)
+    raw, sc, x = synth.uniform_problem(1001, 256, 1024, 1, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    y = gemm_capi(E, M, native, scd, xd, 256)
+    wdq = oracle.dequant(raw, sc, E, M)
+    check_close(y, oracle.gemm(wdq, x).astype(np.float64), "vs fp32-accumulating oracle")
+    check_close(y, oracle.gemm_f64(wdq, x), "vs float64")
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("N", [1, 7, 8, 9, 16, 17, 33, 65, 129, 200])
+def test_batch_edges(E, M, N):
+    print("case batch edge", E, M, N, flush=True)
+    OC, IC = 256, 512
+    raw, sc, x = synth.uniform_problem(300 + N, OC, IC, N, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    y = gemm_capi(E, M, native, scd, xd, OC)
+    assert np.isfinite(y).all()
+    check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "N=%d" % N)
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("splitK", [1, 2, 3, 4, 8, 40])
+def test_split_k(E, M, splitK):
+    """K = 1344 = 5.25 native K blocks; splitK = 40 leaves most splits empty (they must contribute zeros)."""
+    print("case splitK", E, M, splitK, flush=True)
+    OC, IC, N = 256, 1344, 5
+    raw, sc, x = synth.uniform_problem(400 + splitK, OC, IC, N, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    y = gemm_capi(E, M, native, scd, xd, OC, splitK)
+    check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "splitK=%d" % splitK)
+
+
+@pytest.mark.parametrize("cfg", [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 16), (1, 4, 8), (2, 1, 8), (2, 2, 4), (4, 1, 8), (4, 2, 8)])
+def test_every_launch_shape(cfg):
+    print("case launch shape", cfg, flush=True)
+    E, M = 3, 2
+    OC, IC, N = 512, 2304, 16 * cfg[0] - 3
+    raw, sc, x = synth.uniform_problem(500 + sum(cfg), OC, IC, N, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    for splitK in (1, 3):
+        check_close(gemm_capi(E, M, native, scd, xd, OC, splitK, cfg), ref, "cfg %s splitK %d" % (cfg, splitK))
+
+
+def test_unsupported_launch_shape_is_rejected():
+    raw, sc, x = synth.uniform_problem(1, 256, 256, 4)
+    native, scd, xd = upload(raw, sc, x, 3, 2)
+    L = _lib.lib()
+    out = torch.empty((4, 256), dtype=torch.float16, device=DEV)
+    rc = L.fp6mi_linear_native_cfg(3, 2, None, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), 256, 4, 256, None, 1, 3, 1, 8)
+    assert rc == -2
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_known_answers(E, M):
+    """All-ones weights/activations/scales => every output = IC (tests/python/kernel_test_fpx.py:88-131);
+    one-hot activations => a column of the dequantized weights, bit for bit; zero scale => zeros."""
+    ones = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2): [806142768, 3274706115, 214118412]}[(E, M)]
+    OC, IC = 256, 1024
+    words = np.array(ones, dtype=np.uint32)
+    raw = np.tile(words, (OC, IC * (1 + E + M) // 32 // len(words))).view(np.int32)
+    native, scd, xd = upload(raw, np.ones(OC, np.float16), np.ones((8, IC), np.float16), E, M)
+    assert (gemm_capi(E, M, native, scd, xd, OC) == np.float16(IC)).all()
+
+    raw, sc, _ = synth.uniform_problem(77, OC, IC, 1, E, M)
+    x = np.zeros((3, IC), np.float16)
+    x[0, 0], x[1, 517], x[2, IC - 1] = 1, 1, 1
+    native, scd, xd = upload(raw, sc, x, E, M)
+    y = gemm_capi(E, M, native, scd, xd, OC)
+    wdq = oracle.dequant(raw, sc, E, M)
+    for n, k in enumerate((0, 517, IC - 1)):
+        assert (y[n] == wdq[:, k]).all()
+    y0 = gemm_capi(E, M, native, torch.zeros(OC, dtype=torch.float16, device=DEV), xd, OC)
+    assert (y0 == 0).all()
+
+
+# ------------------------------------------------------------------------------------------------ the drop-in API
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_reference_named_api_both_argument_orders(E, M):
+    print("case drop-in api", E, M, flush=True)
+    OC, IC, N = 512, 1024, 8
+    raw, sc, x = synth.uniform_problem(600, OC, IC, N, E, M)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).to(DEV)   # reference layout on the GPU
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    y1 = fp6.linear_forward_eXmY_cuda(E, M, xd, packed, scd, 1)        # order used by the reference's code and tests
+    y2 = fp6.linear_forward_eXmY_cuda(E, M, packed, scd, xd, 2)        # order documented in the reference's README
+    torch.cuda.synchronize()
+    assert y1.shape == (N, OC) and y1.dtype == torch.float16
+    check_close(y1.cpu().numpy(), ref, "code order")
+    check_close(y2.cpu().numpy(), ref, "README order, splitK=2")
+    if (E, M) == (3, 2):
+        y3 = fp6.linear_forward_cuda(xd, packed, scd, 1)
+        assert torch.equal(y3, y1)
+    # an in-place change of the weights must not be served from the cached native copy
+    packed.zero_()
+    y4 = fp6.linear_forward_eXmY_cuda(E, M, xd, packed, scd, 1)
+    assert (y4 == 0).all()
+
+
+# ------------------------------------------------------------------------------------------------ benchmark configs
+def _bench_case(E, M, OC, IC, BS, seed, gaussian, act_sigma=1.0, splitKs=(None,)):
+    print("case bench config", E, M, OC, IC, BS, flush=True)
+    if gaussian:
+        raw, sc, x = synth.gaussian_problem(seed, OC, IC, BS, E, M, act_sigma)
+    else:
+        raw, sc, x = synth.uniform_problem(seed, OC, IC, BS, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    # float64 reference on the CPU from the oracle's dequantized weights, for a sample of output rows at big sizes
+    rows = np.arange(OC) if OC * IC <= 4096 * 4096 else np.sort(np.random.default_rng(seed).choice(OC, 2048, replace=False))
+    sub = quant.pack_raw(quant.unpack_raw(raw[rows], E, M), E, M)
+    wdq = oracle.dequant(sub, sc[rows], E, M)
+    ref = oracle.gemm_f64(wdq, x)
+    for s in splitKs:
+        s = fp6.heuristic_splitk_mi355x(OC, BS, IC) if s is None else s
+        y = gemm_capi(E, M, native, scd, xd, OC, s)
+        check_close(y[:, rows], ref, "%dx%d BS=%d splitK=%d" % (OC, IC, BS, s))
+    return native, scd, xd, raw, sc
+
+
+@pytest.mark.parametrize("BS", [1, 8, 16])
+def test_config2_attention_projection(BS):
+    _bench_case(3, 2, 4096, 4096, BS, 2001, gaussian=False, splitKs=(None, 1, 2, 4, 8))
+
+
+@pytest.mark.parametrize("OC,IC", [(11008, 4096), (4096, 11008)])
+@pytest.mark.parametrize("BS", [8, 32])
+def test_config3_mlp(OC, IC, BS):
+    _bench_case(3, 2, OC, IC, BS, 3001 + (OC > IC), gaussian=True)
+
+
+@pytest.mark.parametrize("OC,IC,seed", [(10240, 8192, 4001), (28672, 8192, 4002), (8192, 28672, 4003)])
+def test_config4_70b_layer(OC, IC, seed):
+    _bench_case(3, 2, OC, IC, 32, seed, gaussian=True, act_sigma=0.5)
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("BS", [1, 2, 4, 8, 16, 32, 64, 128, 256, 512])
+def test_config5_batch_sweep(E, M, BS):
+    if not hasattr(test_config5_batch_sweep, "cache"):
+        test_config5_batch_sweep.cache = {}
+    cache = test_config5_batch_sweep.cache
+    OC = IC = 8192
+    if (E, M) not in cache:
+        cache.clear()
+        raw, sc, _ = synth.gaussian_problem(5001, OC, IC, 1, E, M)
+        rows = np.sort(np.random.default_rng(5).choice(OC, 1024, replace=False))
+        sub = quant.pack_raw(quant.unpack_raw(raw[rows], E, M), E, M)
+        cache[(E, M)] = (fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV), torch.from_numpy(sc).to(DEV), rows,
+                         oracle.dequant(sub, sc[rows], E, M))
+    native, scd, rows, wdq = cache[(E, M)]
+    print("case config5", E, M, BS, flush=True)
+    x = synth.activations(5001 + BS, BS, IC)
+    y = gemm_capi(E, M, native, scd, torch.from_numpy(x).to(DEV), OC)
+    check_close(y[:, rows], oracle.gemm_f64(wdq, x), "8192x8192 BS=%d" % BS)
+
+
+def test_full_size_property_linearity_and_split_invariance():
+    """Size-independent properties at a full benchmark size (28672x8192, BS=32): f(2x) = 2 f(x) exactly, the first 16
+    batch rows computed alone agree with the same rows of the full batch, and split-K 2 agrees with split-K 1."""
+    E, M, OC, IC, BS = 3, 2, 28672, 8192, 32
+    raw, sc, x = synth.gaussian_problem(4002, OC, IC, BS, E, M, 0.5)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    y = gemm_capi(E, M, native, scd, xd, OC)
+    y2 = gemm_capi(E, M, native, scd, xd * 2, OC)
+    normal = np.abs(y.astype(np.float32)) >= 2.0 ** -13      # doubling is exact unless the result is an fp16 subnormal
+    assert normal.mean() > 0.999
+    assert (y2.astype(np.float32)[normal] == 2 * y.astype(np.float32)[normal]).all()
+    # a batch row does not depend on its neighbours; a different batch size only changes the FP32 summation order
+    ya = gemm_capi(E, M, native, scd, xd[:16].contiguous(), OC).astype(np.float64)
+    assert rel_errors(ya, y[:16].astype(np.float64))[0] <= 2e-3
+    ys = gemm_capi(E, M, native, scd, xd, OC, 2).astype(np.float64)
+    mx, _ = rel_errors(ys, y.astype(np.float64))
+    assert mx <= 2e-3

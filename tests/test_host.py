@@ -1,0 +1,209 @@
+"""CPU-side product code (libfp6mi.so through the C ABI and the Python API) against the oracle and the golden fixtures.
+No GPU compute is called here; the library must load and export every symbol that include/fp6mi.h declares."""
+import ctypes
+import glob
+import hashlib
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+import fp6_llm_amd as fp6
+from fp6_llm_amd import _lib, quant, synth
+
+FORMATS = [(3, 2), (2, 2)]
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _problem(seed, OC, IC, E, M):
+    raw, sc, _ = synth.uniform_problem(seed, OC, IC, 1, E, M)
+    return raw, sc
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fp6mi.h")).read()
+    declared = set(re.findall(r"\b(fp6mi_[a-z0-9_]+)\s*\(", header))
+    assert declared and declared == set(_lib.EXPORTED)
+    L = _lib.lib()
+    for name in declared:
+        assert hasattr(L, name), name
+    assert L.fp6mi_version() >= 100
+    assert b"success" in L.fp6mi_error_string(0)
+
+
+def test_golden_prepack_fixtures(golden_dir):
+    for f in sorted(glob.glob(os.path.join(golden_dir, "prepack_e*_*.npz"))):
+        E, M = (3, 2) if "e3m2" in f else (2, 2)
+        z = np.load(f)
+        raw = np.ascontiguousarray(z["raw"])
+        OC, IC = raw.shape[0], raw.shape[1] * 32 // (1 + E + M)
+        got = np.empty_like(raw)   # through the C ABI: the Python wrapper keeps the reference's OC % 256 rule
+        assert _lib.lib().fp6mi_prepack_ref(E, M, got.ctypes.data, raw.ctypes.data, OC, IC) == 0
+        assert got.tobytes() == z["packed"].tobytes(), f
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_prepack_hash_at_benchmark_size(golden_dir, E, M):
+    """Config 2 size (4096x4096): bytes identical to what the reference's prepacker produced (committed SHA-256)."""
+    ref = json.load(open(os.path.join(golden_dir, "prepack_hashes.json")))["e%dm%d_4096x4096_seed2001" % (E, M)]
+    raw = quant.pack_raw(synth.uniform_codes(2001, 4096, 4096, E, M), E, M)
+    assert hashlib.sha256(raw.tobytes()).hexdigest() == ref["raw_sha256"]
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).numpy()
+    assert hashlib.sha256(packed.tobytes()).hexdigest() == ref["packed_sha256"]
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("OC,IC", [(256, 64), (256, 320), (512, 1024)])
+def test_prepack_dequant_native_against_oracle(E, M, OC, IC):
+    raw, sc = _problem(OC + IC, OC, IC, E, M)
+    t = torch.from_numpy(raw)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, t)
+    assert packed.shape == t.shape and packed.dtype == torch.int32
+    assert packed.numpy().tobytes() == oracle.prepack(raw, E, M).tobytes()
+    dq = fp6.weight_dequant_eXmY_cpu(E, M, t, torch.from_numpy(sc)).numpy()
+    assert dq.shape == (OC, IC)
+    assert (dq.view(np.uint16) == oracle.dequant(raw, sc, E, M).view(np.uint16)).all()
+    # native layout: same bits by both routes, and a lossless round trip
+    nat = fp6.weight_prepacking_native_cpu(E, M, t)
+    assert nat.numel() * 4 == fp6.native_bytes(E, M, OC, IC) == (OC // 16) * ((IC + 255) // 256) * (3072 if E == 3 else 2560)
+    assert torch.equal(nat, fp6.to_native(packed, E, M))
+    L = _lib.lib()
+    back = np.empty_like(raw)
+    assert L.fp6mi_unpack_native(E, M, back.ctypes.data, nat.data_ptr(), OC, IC) == 0 and (back == raw).all()
+    back2 = np.empty_like(raw)
+    assert L.fp6mi_unpack_ref(E, M, back2.ctypes.data, packed.data_ptr(), OC, IC) == 0 and (back2 == raw).all()
+
+
+def test_fp6_wrappers_are_the_e3m2_case():
+    raw, sc = _problem(1, 256, 128, 3, 2)
+    t, s = torch.from_numpy(raw), torch.from_numpy(sc)
+    assert torch.equal(fp6.weight_prepacking_cpu(t), fp6.weight_prepacking_eXmY_cpu(3, 2, t))
+    assert torch.equal(fp6.weight_dequant_cpu(t, s), fp6.weight_dequant_eXmY_cpu(3, 2, t, s))
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_native_fp6_lane_image_is_the_hardware_operand(E, M):
+    """Layout spot check written from the layout's definition, not from the packer: row 16R+m, K block U, lane m+16q,
+    code index ci = 8s+j  <->  column 256U + 32s + 8q + j."""
+    x = 1 + E + M
+    OC, IC = 32, 512
+    codes = synth.uniform_codes(42, OC, IC, E, M)
+    nat = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))).numpy().view(np.uint32)
+    bb = (3072 if E == 3 else 2560) // 4
+    for (R, U, lane) in [(0, 0, 0), (1, 1, 37), (0, 1, 63), (1, 0, 16)]:
+        m, q = lane % 16, lane // 16
+        blk = nat[(R * 2 + U) * bb:(R * 2 + U + 1) * bb]
+        want = [codes[16 * R + m, 256 * U + 32 * s + 8 * q + j] for s in range(8) for j in range(8)]
+        if E == 3:
+            d = [blk[(i // 4) * 256 + lane * 4 + i % 4] for i in range(12)]
+            for h in range(2):
+                big = sum(int(d[6 * h + w]) << (32 * w) for w in range(6))
+                got = [(big >> (6 * i)) & 63 for i in range(32)]
+                assert got == [int(v) for v in want[32 * h:32 * h + 32]]
+        else:
+            d = [blk[(i // 4) * 256 + lane * 4 + i % 4] for i in range(8)] + [blk[512 + lane * 2 + i] for i in range(2)]
+            slot = [2, 1, 3, 0]
+            for s in range(8):
+                for p in range(4):
+                    pp = 4 * (s % 4) + p
+                    lo = ((int(d[s]) >> (4 * slot[p])) & 15) | (((int(d[8 + s // 4]) >> (15 - pp)) & 1) << 4)
+                    hi = ((int(d[s]) >> (4 * (slot[p] + 4))) & 15) | (((int(d[8 + s // 4]) >> (31 - pp)) & 1) << 4)
+                    assert (lo, hi) == (int(want[8 * s + 2 * p]), int(want[8 * s + 2 * p + 1]))
+
+
+def test_prepack_in_place_and_padding_is_zero():
+    E, M = 3, 2
+    raw, _ = _problem(9, 256, 320, E, M)
+    L = _lib.lib()
+    buf = raw.copy()
+    assert L.fp6mi_prepack_ref(E, M, buf.ctypes.data, buf.ctypes.data, 256, 320) == 0
+    assert buf.tobytes() == oracle.prepack(raw, E, M).tobytes()
+    # K = 320 is padded to 512 in the native layout: the padded columns hold code 0
+    nat = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw))
+    wide = np.zeros((256, 512), np.uint8)
+    wide[:, :320] = quant.unpack_raw(raw, E, M)
+    assert torch.equal(nat, fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(wide, E, M))))
+
+
+def test_error_codes_instead_of_aborts():
+    L = _lib.lib()
+    buf = np.zeros(1 << 16, np.uint8)
+    p = buf.ctypes.data
+    assert L.fp6mi_prepack_ref(4, 3, p, p, 64, 64) == -1                      # unsupported format (reference: exit(-1))
+    assert L.fp6mi_prepack_ref(3, 2, p, p, 32, 64) == -2                      # M % 64 (reference: assert)
+    assert L.fp6mi_prepack_ref(3, 2, p, p, 64, 96) == -2                      # K % 64
+    assert L.fp6mi_prepack_ref(3, 2, None, p, 64, 64) == -3
+    assert L.fp6mi_dequant(1, 2, p, p, 64, 64, p) == -1
+    assert L.fp6mi_native_bytes(3, 2, 24, 64) == 0
+    assert L.fp6mi_prepack_native(3, 2, p, p, 64, 64) == -2                   # may not alias
+    # GEMM argument checks happen on the host before anything is launched
+    assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 100, 1, 64, None, 1) == -2      # M % 256
+    assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 0, 64, None, 1) == -2      # N == 0
+    assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 1, 96, None, 1) == -2      # K % 64
+    assert L.fp6mi_linear_native(5, 2, None, p, p, p, p, 256, 1, 64, None, 1) == -1
+    assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 1, 64, None, 2) == -4      # splitK without workspace
+    assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 1, 64, None, 0) == -5
+    assert L.fp6mi_linear_native(3, 2, None, None, p, p, p, 256, 1, 64, None, 1) == -3
+    assert L.fp6mi_linear_native(3, 2, None, p + 4, p, p, p, 256, 1, 64, None, 1) == -6  # alignment
+    for code in (-1, -2, -3, -4, -5, -6):
+        assert len(L.fp6mi_error_string(code)) > 8
+    assert L.fp6mi_workspace_bytes(256, 8, 1) == 0 and L.fp6mi_workspace_bytes(256, 8, 3) == 3 * 256 * 8 * 4
+
+
+def test_python_api_argument_errors():
+    t = torch.zeros((256, 12), dtype=torch.int32)
+    with pytest.raises(ValueError):
+        fp6.weight_prepacking_cpu(torch.zeros((100, 12), dtype=torch.int32))      # OC % 256
+    with pytest.raises(ValueError):
+        fp6.weight_prepacking_cpu(torch.zeros((256, 13), dtype=torch.int32))      # width not a multiple of x
+    with pytest.raises(ValueError):
+        fp6.weight_prepacking_cpu(t.to(torch.int64))
+    with pytest.raises(ValueError):
+        fp6.weight_prepacking_eXmY_cpu(4, 3, t)
+    with pytest.raises(ValueError):
+        fp6.weight_dequant_cpu(t, torch.ones(100, dtype=torch.float16))
+    with pytest.raises(ValueError):
+        fp6.linear_forward_cuda(torch.zeros(1, 64, dtype=torch.float16), t, torch.ones(256, dtype=torch.float16), 1)  # not on GPU
+
+
+def test_reference_heuristic_is_kept_verbatim():
+    for args in [(4096, 8, 108), (11008, 8, 108), (8192, 512, 256), (256, 1, 108), (28672, 32, 108), (4096, 8, 256)]:
+        assert fp6.HeuristicFuntion_SplitK(*args) == oracle.heuristic_splitk(*args)
+        assert fp6.Num_Wave(args[0], args[1], 3, args[2]) == pytest.approx(oracle.num_wave(args[0], args[1], 3, args[2]))
+
+
+def test_mi355x_heuristic_prefers_no_split_when_rows_fill_the_chip():
+    for (M, N, K) in [(4096, 8, 4096), (11008, 8, 4096), (8192, 32, 8192), (28672, 32, 8192), (8192, 512, 8192)]:
+        assert fp6.heuristic_splitk_mi355x(M, N, K) == 1
+    s = fp6.heuristic_splitk_mi355x(256, 8, 28672)      # 16 row tiles cannot occupy 256 CUs: splitting K pays
+    assert 2 <= s <= 64
+    assert fp6.heuristic_splitk_mi355x(256, 1, 1024) == 1  # too little work to pay for a second launch
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_quantizer(E, M):
+    x = 1 + E + M
+    mags = quant.magnitudes(E, M)
+    assert (mags == np.abs(oracle.value_table(E, M)[: 1 << (x - 1)])).all()
+    allc = np.arange(1 << x, dtype=np.uint8)
+    vals = oracle.value_table(E, M)
+    q = quant.quantize_codes(vals, E, M)
+    assert (q == allc).all()                                       # exact values map to their own code (incl. -0)
+    assert quant.quantize_codes(np.array([1e9, -1e9]), E, M).tolist() == [(1 << (x - 1)) - 1, (1 << x) - 1]  # clamp
+    mid = (mags[:-1] + mags[1:]) / 2
+    tie = quant.quantize_codes(mid, E, M)
+    assert (tie % 2 == 0).all()                                    # ties go to the even code
+    v = np.linspace(-mags[-1], mags[-1], 4001)
+    assert (np.diff(vals[quant.quantize_codes(v, E, M)]) >= 0).all()  # monotone
+    assert (np.abs(vals[quant.quantize_codes(v, E, M)] - v) <= np.diff(mags).max() / 2 + 1e-12).all()
+    w = synth.normal(5, (64, 128))
+    codes, scale = quant.quantize_rowwise(w, E, M)
+    assert scale.dtype == np.float16 and codes.max() < (1 << x)
+    deq = quant.dequantize_codes(codes, scale, E, M)
+    assert np.abs(deq - w).max() <= np.abs(w).max() / mags[-1] * np.diff(mags).max() * 0.51
+    raw = quant.pack_raw(codes, E, M)
+    assert (quant.unpack_raw(raw, E, M) == codes).all() and (oracle.unpack_codes(raw, E, M) == codes).all()

@@ -1,0 +1,274 @@
+"""Pins the CPU oracle (oracle/) before anything is compared against it.
+
+Each check is chosen so that a plausible mistake in the oracle fails it: fixtures produced by the reference's own
+prepacker, the known-answer constants written in the reference's tests, an independent closed-form index map,
+the format definition evaluated in exact rational arithmetic, and invariants (bijection, in-place == out-of-place).
+"""
+import glob
+import hashlib
+import json
+import os
+import struct
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+import oracle
+from fp6_llm_amd import quant, synth
+
+FORMATS = [(3, 2), (2, 2)]
+# "all weights = 1.0" bit patterns quoted in the reference: tests/python/kernel_test_fpx.py:88-107 (FP5_e2m2) and :110-131 (FP6_e3m2)
+ONES = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2): [806142768, 3274706115, 214118412]}
+
+
+def _ones_raw(E, M, OC, IC):
+    words = np.array(ONES[(E, M)], dtype=np.uint32)
+    reps = IC // (32 * len(words) // (1 + E + M))
+    return np.tile(words, (OC, reps)).view(np.int32)
+
+
+# ------------------------------------------------------------------------------------------------ raw format
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_all_ones_pattern_decodes_to_the_code_of_one(E, M):
+    # 1.0 = sign 0, exponent = bias, mantissa 0: e3m2 -> 0 011 00 = 12, e2m2 -> 0 01 00 = 4 (kernel_test_fpx.py:102,125)
+    raw = _ones_raw(E, M, 64, 128)
+    codes = oracle.unpack_codes(raw, E, M)
+    assert set(np.unique(codes)) == {12 if E == 3 else 4}
+    assert (oracle.raw_to_codes(raw, E, M) == codes).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_bitstream_is_msb_first(E, M):
+    x = 1 + E + M
+    codes = np.zeros((64, 64), dtype=np.uint8)
+    codes[0, 0] = (1 << x) - 1      # first code all ones -> top x bits of byte 0
+    codes[0, 1] = 1                 # second code = 1 -> its LSB is bit 2x-1 of the stream
+    raw = oracle.codes_to_raw(codes, E, M)
+    assert raw[0, 0] >> (8 - x) == (1 << x) - 1
+    bit = 2 * x - 1
+    assert (raw[0, bit // 8] >> (7 - bit % 8)) & 1 == 1
+    assert (oracle.unpack_codes(raw, E, M) == codes).all()
+
+
+# ------------------------------------------------------------------------------------------------ prepacking
+def test_golden_prepack_fixtures(golden_dir):
+    files = sorted(glob.glob(os.path.join(golden_dir, "prepack_e*_*.npz")))
+    assert len(files) == 6
+    for f in files:
+        E, M = (3, 2) if "e3m2" in f else (2, 2)
+        z = np.load(f)
+        got = oracle.prepack(z["raw"], E, M)
+        assert got.tobytes() == z["packed"].tobytes(), f
+        # the fixture's input is what the generator produces from its seed (fixtures are reproducible)
+        OC = z["raw"].shape[0]
+        IC = z["raw"].shape[1] * 32 // (1 + E + M)
+        assert (quant.pack_raw(synth.uniform_codes(int(z["seed"]), OC, IC, E, M), E, M) == z["raw"]).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_golden_hash_config1(golden_dir, E, M):
+    name = "e%dm%d_256x1024_seed1001" % (E, M)
+    ref = json.load(open(os.path.join(golden_dir, "prepack_hashes.json")))[name]
+    raw = quant.pack_raw(synth.uniform_codes(1001, 256, 1024, E, M), E, M)
+    assert hashlib.sha256(raw.tobytes()).hexdigest() == ref["raw_sha256"]
+    assert hashlib.sha256(oracle.prepack(raw, E, M).tobytes()).hexdigest() == ref["packed_sha256"]
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_prepack_matches_reference_build_when_present(E, M):
+    if oracle.ref_lib() is None:
+        pytest.skip("oracle/_ref not built on this machine")
+    rng = np.random.default_rng(5)
+    raw = rng.integers(0, 256, size=(192, 128 * (1 + E + M) // 8), dtype=np.uint8)
+    assert (oracle.prepack(raw, E, M) == oracle.ref_prepack(raw, E, M)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_prepack_closed_form_index_map(E, M):
+    x = 1 + E + M
+    rng = np.random.default_rng(7)
+    codes = rng.integers(0, 1 << x, size=(128, 192), dtype=np.uint8)
+    raw = oracle.codes_to_raw(codes, E, M)
+    assert (oracle.prepack(raw, E, M) == oracle.prepack_closed_form(codes, E, M)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_prepack_all_ones_known_answer(E, M):
+    # 1.0 splits into an all-zero high segment and the nibble 1100 (e3m2) / 0100 (e2m2) in every 4-bit fragment
+    raw = _ones_raw(E, M, 64, 128)
+    words = oracle.prepack(raw, E, M).view(np.uint32).reshape(-1)
+    hi_words = 64 * 128 * (2 if E == 3 else 1) // 32
+    assert (words[:hi_words] == 0).all()
+    assert (words[hi_words:] == (0xCCCCCCCC if E == 3 else 0x44444444)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_prepack_is_a_bit_permutation_and_in_place_safe(E, M):
+    x = 1 + E + M
+    rng = np.random.default_rng(9)
+    raw = rng.integers(0, 256, size=(64, 64 * x // 8), dtype=np.uint8)
+    packed = oracle.prepack(raw, E, M)
+    assert np.unpackbits(raw).sum() == np.unpackbits(packed).sum()
+    # one-hot inputs map to one-hot outputs at distinct positions (bijection on bits), sampled
+    seen = set()
+    for bit in range(0, raw.size * 8, 97):
+        one = np.zeros(raw.size, dtype=np.uint8)
+        one[bit // 8] = 0x80 >> (bit % 8)
+        out = np.unpackbits(oracle.prepack(one.reshape(raw.shape), E, M))
+        assert out.sum() == 1
+        seen.add(int(out.argmax()))
+    assert len(seen) == len(range(0, raw.size * 8, 97))
+    # aliased call
+    buf = raw.copy()
+    rc = oracle.lib().orc_prepack(E, M, buf.ctypes.data, buf.ctypes.data, 64, 64)
+    assert rc == 0 and (buf == packed).all()
+
+
+def test_prepack_rejects_what_the_reference_asserts():
+    raw = np.zeros((32, 48), dtype=np.uint8)
+    with pytest.raises(ValueError):
+        oracle.prepack(raw, 3, 2)              # rows % 64
+    with pytest.raises(ValueError):
+        oracle.prepack(np.zeros((64, 48), np.uint8), 4, 3)  # unsupported format
+
+
+# ------------------------------------------------------------------------------------------------ dequantisation
+def _half_bits_of_fraction(v):
+    """IEEE binary16 bits of an exact rational, rounded to nearest even by Python's own packer ('e' format)."""
+    return struct.unpack("<H", struct.pack("<e", float(v)))[0]  # float(v) is exact here: <= 14 significant bits
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_format_constants(E, M):
+    tab = oracle.value_table(E, M)
+    x = 1 + E + M
+    if E == 3:  # utils/weight_quant.h:22-25: max 28, smallest subnormal 0.0625
+        assert tab[0b011111] == 28.0 and tab[0b000001] == 0.0625 and tab[0b001100] == 1.0
+    else:
+        assert tab[0b01111] == 7.0 and tab[0b00001] == 0.25 and tab[0b00100] == 1.0
+    assert (tab[(1 << (x - 1)):] == -tab[: (1 << (x - 1))]).all()
+    assert np.signbit(tab[1 << (x - 1)]) and tab[1 << (x - 1)] == 0.0   # negative zero exists
+    assert np.isfinite(tab).all()                                       # exponent all-ones is an ordinary value
+    assert (np.diff(tab[: (1 << (x - 1))]) > 0).all()                   # magnitude code order is value order
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_dequant_all_ones_is_one(E, M):
+    raw = _ones_raw(E, M, 64, 128)
+    out = oracle.dequant(raw, np.ones(64, np.float16), E, M)
+    assert (out == np.float16(1.0)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_dequant_exhaustive_codes_times_scale_samples(E, M):
+    """Every code against ~4000 fp16 scales spread over the whole fp16 range (normals, subnormals, zero, big values that
+    overflow to inf), checked against the format definition in exact arithmetic."""
+    x = 1 + E + M
+    ncodes = 1 << x
+    scale_bits = np.unique(np.concatenate([np.arange(0, 0x7C00, 8), [1, 2, 3, 0x03FF, 0x0400, 0x3C00, 0x7BFF, 0x8001, 0xBC00, 0xFBFF]]))
+    scale_bits = scale_bits[: (len(scale_bits) // 64) * 64].astype(np.uint16)
+    scales = scale_bits.view(np.float16)
+    K = 64
+    codes = np.tile(np.arange(ncodes, dtype=np.uint8), K // ncodes if ncodes <= K else 1)
+    codes = np.resize(np.arange(ncodes, dtype=np.uint8), K)[None, :].repeat(len(scales), axis=0)
+    raw = oracle.codes_to_raw(codes, E, M)
+    got = oracle.dequant(raw, scales, E, M).view(np.uint16)
+    # numpy float64 path (exact product, one rounding) for all entries
+    want = oracle.dequant_from_definition(codes, scales, E, M).view(np.uint16)
+    assert (got == want).all()
+    # and, for a sample, pure-Python rationals rounded by struct's binary16 packer (shares nothing with numpy)
+    for r in range(0, len(scales), 37):
+        s = Fraction(float(scales[r]))
+        for c in range(ncodes):
+            v = oracle.value_of_code(int(codes[r, c % K]), E, M) * s
+            if abs(v) >= 65520:
+                want_bits = 0x7C00 | (0x8000 if v < 0 else 0)
+            else:
+                want_bits = _half_bits_of_fraction(v)
+                if v == 0 and ((codes[r, c % K] >> (x - 1)) ^ (scale_bits[r] >> 15)) & 1:
+                    want_bits |= 0x8000
+            assert got[r, c % K] == want_bits, (r, c, float(scales[r]))
+
+
+def test_half_conversion_helpers_against_numpy():
+    L = oracle.lib()
+    rng = np.random.default_rng(3)
+    vals = np.concatenate([rng.standard_normal(2000).astype(np.float32) * np.float32(10.0) ** rng.integers(-8, 5, 2000),
+                           np.array([0.0, -0.0, 65504.0, 65519.9, 65520.0, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 6.1e-5], np.float32)])
+    for v in vals:
+        assert L.orc_float_to_half(float(v)) == np.float32(v).astype(np.float16).view(np.uint16), v
+    for h in range(0, 0x7C00, 13):
+        assert L.orc_half_to_float(h) == float(np.uint16(h).view(np.float16))
+
+
+# ------------------------------------------------------------------------------------------------ split-K, launcher logic
+@pytest.mark.parametrize("K,s", [(64, 1), (4096, 3), (4096, 13), (1024, 16), (1024, 17), (11008, 5), (256, 8)])
+def test_splitk_partition_closed_form(K, s):
+    nb = K // 64
+    ranges = [oracle.splitk_range(K, s, i) for i in range(s)]
+    pos = 0
+    for i, (start, n) in enumerate(ranges):
+        assert start == pos
+        assert n == nb // s + (1 if i < nb % s else 0)   # first nb % s splits are one block longer
+        pos += n
+    assert pos == nb
+
+
+def test_splitk_reduce_sums_in_split_order():
+    ws = np.zeros((3, 2, 256), dtype=np.float32)
+    ws[0] += 1e8
+    ws[1] += 1.0
+    ws[2] -= 1e8
+    out = oracle.splitk_reduce(ws)   # (1e8 + 1) - 1e8 in fp32 = 0, not 1: order matters
+    assert (out == 0).all()
+    ws2 = np.random.default_rng(1).standard_normal((4, 3, 256)).astype(np.float32)
+    want = ((ws2[0] + ws2[1]) + ws2[2]) + ws2[3]
+    assert (oracle.splitk_reduce(ws2) == want.astype(np.float16)).all()
+
+
+def test_tile_n_buckets():
+    # fp6_linear.cu:61-75
+    assert [oracle.tile_n(n) for n in (1, 8, 9, 16, 17, 32, 33, 64, 65, 128, 129, 1000)] == [8, 8, 16, 16, 32, 32, 64, 64, 64, 64, 64, 64]
+
+
+def test_heuristic_known_answers():
+    # hand-evaluated from fp6_llm/__init__.py:6-23
+    known = {(4096, 8, 108): 11, (11008, 8, 108): 4, (10240, 32, 108): 5, (28672, 32, 108): 5, (8192, 32, 108): 6,
+             (8192, 128, 108): 3, (8192, 512, 108): 3, (4096, 8, 256): 26, (11008, 8, 256): 10, (8192, 32, 256): 13,
+             (8192, 512, 256): 2, (256, 1, 256): 1, (256, 1, 108): 87}
+    for args, want in known.items():
+        assert oracle.heuristic_splitk(*args) == want, args
+    # 4096x8 on 108 SMs: ceil(4096/512)=8 CTAs per split; 11 splits -> 88/108 = 0.815 of one wave, 10 -> 0.74
+    assert abs(oracle.num_wave(4096, 8, 11, 108) - 88 / 108) < 1e-12
+
+
+# ------------------------------------------------------------------------------------------------ GEMM definition
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_gemm_special_cases(E, M):
+    OC, IC = 64, 128
+    ones = _ones_raw(E, M, OC, IC)
+    wdq = oracle.dequant(ones, np.ones(OC, np.float16), E, M)
+    out = oracle.gemm(wdq, np.ones((3, IC), np.float16))
+    assert (out == np.float16(IC)).all()                     # all ones => every output = IC (kernel_test_fpx.py:98-99)
+    # one-hot activations pick a column of the dequantized weights exactly
+    raw, sc, _ = synth.uniform_problem(3, OC, IC, 1, E, M)
+    wdq = oracle.dequant(raw, sc, E, M)
+    x = np.zeros((2, IC), np.float16)
+    x[0, 5] = 1
+    x[1, 77] = 1
+    out = oracle.gemm(wdq, x)
+    # (value equality: a negative-zero weight sums to +0)
+    assert (out[0] == wdq[:, 5]).all() and (out[1] == wdq[:, 77]).all()
+
+
+def test_gemm_against_float64_and_split_k():
+    raw, sc, x = synth.uniform_problem(11, 64, 256, 5)
+    wdq = oracle.dequant(raw, sc)
+    ref = oracle.gemm_f64(wdq, x)
+    for s in (1, 2, 3, 4, 7):
+        out = oracle.gemm(wdq, x, s).astype(np.float64)
+        den = np.maximum(np.abs(ref), np.sqrt((ref ** 2).mean()))
+        assert (np.abs(out - ref) / den).max() < 2e-3
+    with pytest.raises(ValueError):
+        oracle.gemm(wdq, x, 0)
