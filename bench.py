@@ -1,0 +1,266 @@
+#!/usr/bin/env python3
+"""Benchmark of the FPx x FP16 linear layer on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--sweep]
+
+A step is one GEMM of the workload (default: the headline one, FP6_e3m2 4096x4096, batch 8, split-K from the engine's
+heuristic).  Weights are synthetic, already resident in HBM, and ROTATE through a pool of distinct buffers larger than the
+256 MB last-level cache, so every step streams its weights from HBM like consecutive layers of a model would ("cold");
+the same-buffer ("warm") figure is reported beside it.  The K steps are captured once into a HIP graph and replayed inside
+the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 us kernel.
+
+Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth figure the reference's design is judged
+on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
+launch stream; `cpu_baseline` times the reference's CPU path (dequantize, then a torch CPU matmul) on this host.
+--sweep additionally runs every benchmark configuration and writes gpurun_out/bench_sweep.jsonl.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 MFMA
+POOL_BYTES = 1 << 30            # distinct weight buffers cycled through: 4x the 256 MB last-level cache
+
+WORKLOADS = {
+    # name: (E, M, OC, IC, BS)
+    "fp6_4096x4096_bs8": (3, 2, 4096, 4096, 8),
+    "fp6_4096x4096_bs1": (3, 2, 4096, 4096, 1),
+    "fp6_4096x4096_bs16": (3, 2, 4096, 4096, 16),
+    "fp6_11008x4096_bs8": (3, 2, 11008, 4096, 8),
+    "fp6_11008x4096_bs32": (3, 2, 11008, 4096, 32),
+    "fp6_4096x11008_bs8": (3, 2, 4096, 11008, 8),
+    "fp6_4096x11008_bs32": (3, 2, 4096, 11008, 32),
+    "fp6_10240x8192_bs32": (3, 2, 10240, 8192, 32),
+    "fp6_28672x8192_bs32": (3, 2, 28672, 8192, 32),
+    "fp6_8192x28672_bs32": (3, 2, 8192, 28672, 32),
+}
+for _bs in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
+    WORKLOADS["fp6_8192x8192_bs%d" % _bs] = (3, 2, 8192, 8192, _bs)
+    WORKLOADS["fp5_8192x8192_bs%d" % _bs] = (2, 2, 8192, 8192, _bs)
+HEADLINE = "fp6_4096x4096_bs8"
+
+
+def weight_bytes(E, M, OC, IC):
+    return OC * IC * (1 + E + M) // 8
+
+
+def algorithmic_bytes(E, M, OC, IC, BS):
+    """weights + scales + activations once + output once"""
+    return weight_bytes(E, M, OC, IC) + 2 * OC + 2 * BS * IC + 2 * BS * OC
+
+
+class Problem:
+    """Device buffers of one workload: a pool of native-layout weight buffers, scales, activations, output, workspace."""
+
+    def __init__(self, E, M, OC, IC, BS, device):
+        import torch
+        import fp6_llm_amd as fp6
+        from fp6_llm_amd import quant, synth
+
+        self.E, self.M, self.OC, self.IC, self.BS = E, M, OC, IC, BS
+        self.splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC)
+        nbytes = fp6.native_bytes(E, M, OC, IC)
+        self.nbuf = int(max(2, min(128, POOL_BYTES // nbytes)))
+        # distinct buffers, distinct contents: uniform random codes (every bit pattern is a valid weight)
+        self.weights = []
+        rows = min(OC, 1024)
+        block = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(synth.uniform_codes(2001, rows, IC, E, M), E, M)))
+        reps = OC // rows + (1 if OC % rows else 0)
+        base = block.repeat(reps)[: nbytes // 4].contiguous()
+        for i in range(self.nbuf):
+            self.weights.append(torch.roll(base, shifts=257 * i).to(device))
+        self.scales = torch.from_numpy(synth.uniform_scales(2001, OC)).to(device)
+        self.x = torch.from_numpy(synth.activations(2001, BS, IC)).to(device)
+        self.out = torch.empty((BS, OC), dtype=torch.float16, device=device)
+        self.ws = torch.empty(self.splitK * BS * OC, dtype=torch.float32, device=device) if self.splitK > 1 else None
+
+    def step(self, i, cold=True):
+        import fp6_llm_amd as fp6
+
+        w = self.weights[i % self.nbuf] if cold else self.weights[0]
+        fp6.linear_forward_native(self.E, self.M, self.x, w, self.scales, self.OC, self.splitK, out=self.out, workspace=self.ws)
+
+
+def time_steps(prob, steps, warmup, cold):
+    """Returns (wall seconds between the two synchronizations, HIP-event milliseconds on the launch stream)."""
+    import torch
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            prob.step(i, cold)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(steps):
+                prob.step(warmup + i, cold)
+        graph.replay()  # untimed: first replay uploads the graph
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        t0 = time.perf_counter()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+    return t1 - t0, e0.elapsed_time(e1)
+
+
+def fp16_baseline_us(prob, steps, warmup):
+    """FP16 GEMM of the same shape on the same GPU (torch F.linear = hipBLASLt/rocBLAS), weights rotating the same way:
+    the counterpart of the reference's cuBLAS baseline (tests/python/kernel_test_fp6.py:45-62)."""
+    import torch
+
+    dev = prob.x.device
+    nb = prob.OC * prob.IC * 2
+    nbuf = int(max(2, min(64, POOL_BYTES // nb)))
+    ws = [torch.randn(prob.OC, prob.IC, dtype=torch.float16, device=dev) for _ in range(nbuf)]
+    for i in range(warmup):
+        torch.nn.functional.linear(prob.x, ws[i % nbuf])
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        torch.nn.functional.linear(prob.x, ws[0])
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    torch.nn.functional.linear(prob.x, ws[i % nbuf])
+            graph.replay()
+            torch.cuda.synchronize()
+            e0.record()
+            graph.replay()
+            e1.record()
+        except RuntimeError:  # the BLAS library refused capture: time plain launches instead
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(steps):
+                torch.nn.functional.linear(prob.x, ws[i % nbuf])
+            e1.record()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
+def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
+    """The reference's CPU path on this host: weight_dequant_cpu (utils/weight_dequant.h:10-48, restated by the scalar C
+    oracle, one thread) followed by a torch CPU fp16 matmul (tests/python/kernel_test_fp6.py:48-58 on the CPU)."""
+    import torch
+
+    import oracle
+    from fp6_llm_amd import quant, synth
+
+    raw = quant.pack_raw(synth.uniform_codes(2001, OC, IC, E, M), E, M)
+    sc = synth.uniform_scales(2001, OC)
+    x = torch.from_numpy(synth.activations(2001, BS, IC))
+    reps, t_total, t_deq, t_mm = 0, 0.0, 0.0, 0.0
+    while reps < 3 or (t_total < budget_s and reps < 50):
+        t0 = time.perf_counter()
+        w = torch.from_numpy(oracle.dequant(raw, sc, E, M))
+        t1 = time.perf_counter()
+        torch.nn.functional.linear(x, w)
+        t2 = time.perf_counter()
+        reps += 1
+        t_deq += t1 - t0
+        t_mm += t2 - t1
+        t_total += t2 - t0
+    per = t_total / reps
+    return {
+        "value": round(weight_bytes(E, M, OC, IC) / per / 1e9, 4), "unit": "GB/s", "cores": int(torch.get_num_threads()), "kind": "port",
+        "sample": "%d x (oracle dequant %dx%d on 1 thread: %.1f ms + torch CPU fp16 F.linear BS=%d on %d threads: %.2f ms); host has %d cpus"
+                  % (reps, OC, IC, t_deq / reps * 1e3, BS, torch.get_num_threads(), t_mm / reps * 1e3, os.cpu_count()),
+        "us_per_gemm": round(per * 1e6, 1),
+    }
+
+
+def run_workload(name, steps, warmup, device, with_fp16=True):
+    E, M, OC, IC, BS = WORKLOADS[name]
+    prob = Problem(E, M, OC, IC, BS, device)
+    wall_s, ev_ms = time_steps(prob, steps, warmup, cold=True)
+    _, ev_ms_warm = time_steps(prob, steps, warmup, cold=False)
+    us = ev_ms * 1e3 / steps
+    us_warm = ev_ms_warm * 1e3 / steps
+    wb = weight_bytes(E, M, OC, IC)
+    flops = 2.0 * OC * IC * BS
+    res = {
+        "workload": name, "us_per_gemm": round(us, 3), "us_per_gemm_wall": round(wall_s * 1e6 / steps, 3), "us_per_gemm_warm": round(us_warm, 3),
+        "weight_GBps": round(wb / us / 1e3, 1), "weight_GBps_warm": round(wb / us_warm / 1e3, 1), "tflops": round(flops / us / 1e6, 2),
+        "hbm_frac": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
+        "splitK": prob.splitK, "weight_buffers": prob.nbuf, "weight_bytes": wb, "algorithmic_bytes": algorithmic_bytes(E, M, OC, IC, BS),
+    }
+    if with_fp16:
+        del prob.weights[2:]
+        import torch
+        torch.cuda.empty_cache()
+        f16 = fp16_baseline_us(prob, min(steps, 200), min(warmup, 10))
+        res["fp16_gemm_us"] = round(f16, 3)
+        res["speedup_vs_fp16"] = round(f16 / us, 3)
+    return res, wall_s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
+    ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration (writes gpurun_out/bench_sweep.jsonl)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        sys.exit("bench.py: this path runs on ONE GPU (a linear layer shards by output rows without any collective); use --gpus 1")
+
+    import torch
+
+    import fp6_llm_amd  # noqa: F401  (raises if libfp6mi.so is missing: there is no fallback)
+
+    assert torch.cuda.is_available(), "bench.py needs the GPU"
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    if args.calibrate_copy:
+        src = torch.empty(64 << 20, dtype=torch.uint8, device=device).random_()
+        dst = torch.empty_like(src)
+        for _ in range(10):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy)
+    E, M, OC, IC, BS = WORKLOADS[args.workload]
+    line = {
+        "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["us_per_gemm"] / 1e3, 6),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "%s: FP%d_e%dm2 weights [%d,%d] x fp16 activations [%d,%d], weights rotating through %d distinct HBM buffers, splitK=%d"
+                               % (args.workload, 1 + E + M, E, OC, IC, BS, IC, res["weight_buffers"], res["splitK"])},
+        "roofline": {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"], "traffic": None,
+                     "bytes_per_launch": res["weight_bytes"], "kernel_us": res["us_per_gemm"]},
+        "detail": res,
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline(E, M, OC, IC, BS)
+    if args.sweep:
+        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
+        with open(os.path.join(ROOT, "gpurun_out", "bench_sweep.jsonl"), "w") as f:
+            for name in WORKLOADS:
+                big = WORKLOADS[name][2] * WORKLOADS[name][3] > 64e6
+                r, _ = run_workload(name, 100 if big else 300, 10, device)
+                f.write(json.dumps(r) + "\n")
+                f.flush()
+                print("%-22s %8.2f us  %7.0f GB/s (%.1f%% HBM)  %7.1f TFLOP/s  fp16 %8.2f us  x%.2f" % (
+                    name, r["us_per_gemm"], r["weight_GBps"], 100 * r["hbm_frac"], r["tflops"], r["fp16_gemm_us"], r["speedup_vs_fp16"]), file=sys.stderr, flush=True)
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()
