@@ -36,7 +36,7 @@ def lib():
         "fp6mi_heuristic_splitk": (ci, [sz, sz, sz, ci]),
         "fp6mi_workspace_bytes": (sz, [sz, sz, ci]),
         "fp6mi_linear_native": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci]),
-        "fp6mi_linear_native_cfg": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci, ci, ci, ci]),
+        "fp6mi_linear_native_cfg": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci, ci, ci, ci, ci, ci]),
         "fp6mi_relayout_ref_to_native_gpu": (ci, [ci, ci, vp, vp, vp, sz, sz]),
         "fp6mi_dequant_native_gpu": (ci, [ci, ci, vp, vp, vp, vp, sz, sz]),
     }

@@ -233,6 +233,192 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     }
 }
 
+// A operands of MFMA steps 4h..4h+3 (half of a K block) of one lane.
+__device__ __forceinline__ void convert_half(const WFrag<6> &f, int h, v8h (&o)[4])
+{
+    v6u src = h == 0 ? (v6u){ f.a[0], f.a[1], f.a[2], f.a[3], f.b[0], f.b[1] } : (v6u){ f.b[2], f.b[3], f.c[0], f.c[1], f.c[2], f.c[3] };
+    v32h v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
+#pragma unroll
+    for (int i = 0; i < 4; i++) o[i] = slice8(v, i);
+}
+__device__ __forceinline__ void convert_half(const WFrag<5> &f, int h, v8h (&o)[4])
+{
+    constexpr uint32_t kNib = 0x0F000F00u, kSign = 0x80008000u;
+    const v4u          nib = h == 0 ? f.a : f.b;
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+        uint32_t w = nib[i], sg = f.s[h] << (4 * i);
+        v4u      r;
+        r[0] = (w & kNib) | (sg & kSign);
+        r[1] = ((w << 4) & kNib) | ((sg << 1) & kSign);
+        r[2] = ((w >> 4) & kNib) | ((sg << 2) & kSign);
+        r[3] = ((w << 8) & kNib) | ((sg << 3) & kSign);
+        o[i] = __builtin_bit_cast(v8h, r);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gemm_tile: GEMM for batches above 16, where every weight must meet many activation columns.
+//   workgroup = WR x WK wavefronts; tile = (WR*RT*16) rows x (NT*16) columns
+//   grid.x enumerates (row block, column block, split) with column blocks of one row block adjacent on one XCD
+// The K blocks of a split are walked in chunks of WK blocks.  Per chunk the workgroup stages the activation chunk
+// [WK][NT*16][256] in LDS (double-buffered, filled by fully coalesced 16-byte loads); wavefront (wr, wk) streams the
+// weights of its RT row tiles for K block wk straight from HBM into VGPRs (prefetched one chunk ahead), converts them
+// half a block at a time and runs RT*NT MFMAs per step against B operands read once per step from LDS.  The LDS row
+// stride is 256+8 halfs so that the eight lanes that read 16 bytes each in one LDS cycle fall in distinct banks.
+// The WK partial accumulators are summed through LDS at the end (WK > 1), then scaled and stored.
+// ---------------------------------------------------------------------------------------------------------------
+constexpr int kXsRowBytes = 528;
+
+template <int XB, int NT, int RT, int WR, int WK>
+__global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
+                                                           const half_t *__restrict__ X, half_t *__restrict__ C,
+                                                           float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
+                                                           uint32_t units, uint32_t splitK, uint32_t nblocks)
+{
+    constexpr int  TN = NT * 16, NTHREADS = WR * WK * kWave;
+    constexpr int  kBufBytes = WK * TN * kXsRowBytes;
+    constexpr int  kPieces = WK * TN * 32, kPerThread = (kPieces + NTHREADS - 1) / NTHREADS;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int wr = wave % WR, wk = wave / WR;
+    const int col = lane & 15, q = lane >> 4;
+
+    // grid.x -> (row block, column block, split): ids that are congruent mod 8 run on one XCD and share its L2, so
+    // the column blocks of a row block (which read the same weights) are given such ids
+    uint32_t id = blockIdx.x;
+    if ((gridDim.x & 7u) == 0) id = (id & 7u) * (gridDim.x >> 3) + (id >> 3);
+    const uint32_t nb = id % nblocks, rest = id / nblocks, split = rest % splitK, mb = rest / splitK;
+    const uint32_t nbase = nb * TN, R0 = (mb * WR + wr) * RT; // first row tile of this wavefront
+
+    const uint32_t avg = units / splitK, extra = units % splitK;
+    const uint32_t u0 = split * avg + (split < extra ? split : extra);
+    const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
+
+    const size_t   tile_stride = (size_t)units * Fmt<XB>::block_bytes;
+    const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
+
+    v4f acc[RT][NT];
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+
+    WFrag<XB> wcur[RT], wnxt[RT];
+    v4u       xr[kPerThread];
+
+    auto load_w = [&](WFrag<XB>(&dst)[RT], uint32_t c0) {
+        const uint32_t u = c0 + wk;
+        if (u < u1) {
+#pragma unroll
+            for (int r = 0; r < RT; r++) dst[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
+        }
+    };
+    auto load_x = [&](uint32_t c0) {
+#pragma unroll
+        for (int j = 0; j < kPerThread; j++) {
+            const uint32_t p = tid + NTHREADS * j;
+            v4u            z = { 0, 0, 0, 0 };
+            xr[j]            = z;
+            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
+                const uint32_t k = (c0 + p / (TN * 32)) * 256 + (p & 31) * 8, n = nbase + (p >> 5) % TN;
+                if (n < N && k < K && c0 + p / (TN * 32) < u1) xr[j] = *reinterpret_cast<const v4u *>(X + (size_t)n * K + k);
+            }
+        }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < kPerThread; j++) {
+            const uint32_t p = tid + NTHREADS * j;
+            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces)
+                *reinterpret_cast<v4u *>(lds + buf * kBufBytes + (p >> 5) * kXsRowBytes + (p & 31) * 16) = xr[j];
+        }
+    };
+
+    if (u0 < u1) {
+        load_x(u0);
+        load_w(wcur, u0);
+        store_x(0);
+        __syncthreads();
+        int buf = 0;
+        for (uint32_t c0 = u0; c0 < u1; c0 += WK, buf ^= 1) {
+            const bool more = c0 + WK < u1;
+            if (more) {
+                load_x(c0 + WK);
+                load_w(wnxt, c0 + WK);
+            }
+            if (c0 + wk < u1) {
+                const uint8_t *xs = lds + buf * kBufBytes + (wk * TN + col) * kXsRowBytes + q * 16;
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    v8h a[RT][4];
+#pragma unroll
+                    for (int r = 0; r < RT; r++) convert_half(wcur[r], h, a[r]);
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        v8h b[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xs + t * 16 * kXsRowBytes + (4 * h + s) * 64);
+#pragma unroll
+                        for (int r = 0; r < RT; r++)
+#pragma unroll
+                            for (int t = 0; t < NT; t++) acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[r][s], b[t], acc[r][t], 0, 0, 0);
+                    }
+                }
+            }
+            if (more) {
+                store_x(buf ^ 1); // that buffer was last read before the barrier that ended the previous iteration
+#pragma unroll
+                for (int r = 0; r < RT; r++) wcur[r] = wnxt[r];
+            }
+            __syncthreads();
+        }
+    }
+
+    // acc[r][t][i]: output row (R0+r)*16 + 4q+i, batch column nbase + 16t + col
+    if (WK > 1) {
+        float *red = reinterpret_cast<float *>(lds); // [WK][WR][RT*NT][256]; the last barrier above freed the buffers
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[(((wk * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]) = acc[r][t];
+        __syncthreads();
+        if (wk == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; r++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int k2 = 1; k2 < WK; k2++)
+                        acc[r][t] += *reinterpret_cast<const v4f *>(&red[(((k2 * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]);
+        }
+    }
+    if (wk == 0) {
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+            const uint32_t mg = (R0 + r) * 16 + 4 * q;
+            typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+            const v4h sc4 = *reinterpret_cast<const v4h *>(scales + mg);
+#pragma unroll
+            for (int t = 0; t < NT; t++) {
+                const uint32_t ng = nbase + 16 * t + col;
+                if (ng < N) {
+                    v4f v;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[i] * Fmt<XB>::post_scale);
+                    if (splitK == 1) {
+                        v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
+                        *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
+                    } else {
+                        *reinterpret_cast<v4f *>(ws + ((size_t)split * N + ng) * M + mg) = v;
+                    }
+                }
+            }
+        }
+    }
+}
+
 // C[i] = fp16_rn(sum over splits, in split order, of ws[s][i]); four outputs per thread.
 __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK)
 {
@@ -372,49 +558,120 @@ int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, 
     return (int)hipGetLastError();
 }
 
-struct StreamCfg { int nt, rt, waves; };
-
-// Launch shape of the stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M
-// as long as M/(16*rt) workgroups still cover the compute units; wavefronts per workgroup follow the K blocks available
-// to one split and the register budget (16 wavefronts leave 128 VGPRs each).
-inline StreamCfg pick_cfg(size_t M, size_t N, size_t K, int splitK, int cus)
+template <int XB, int NT, int RT, int WR, int WK>
+int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K, int splitK)
 {
-    StreamCfg c;
-    c.nt = N <= 16 ? 1 : N <= 32 ? 2 : 4;
-    size_t tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
-    size_t nblk = (N + 16 * c.nt - 1) / (16 * c.nt);
-    c.rt = 1;
-    int max_rt = c.nt == 1 ? 4 : 2;
-    while (c.rt < max_rt && tiles % (2 * c.rt) == 0 && (tiles / (2 * c.rt)) * splitK * nblk >= (size_t)cus) c.rt *= 2;
-    int max_waves = (c.nt == 1 && c.rt <= 2) ? 16 : 8;
-    c.waves = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
-    if (c.waves > max_waves) c.waves = max_waves;
+    constexpr int TN = NT * 16, TM = WR * RT * 16;
+    constexpr size_t x_bytes = 2 * (size_t)WK * TN * kXsRowBytes, red_bytes = WK > 1 ? (size_t)WK * WR * RT * NT * 1024 : 0;
+    constexpr size_t lds_bytes = x_bytes > red_bytes ? x_bytes : red_bytes;
+    static_assert(lds_bytes <= 160 * 1024, "tile does not fit in LDS");
+    if (M % TM) return FP6MI_ERR_SHAPE;
+    static bool attr_set = false; // idempotent, so a race between host threads is harmless
+    if (!attr_set && lds_bytes > 48 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<XB, NT, RT, WR, WK>),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if (e != hipSuccess) return (int)e;
+        attr_set = true;
+    }
+    uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
+    size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
+    if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
+    hipLaunchKernelGGL((gemm_tile<XB, NT, RT, WR, WK>), dim3((uint32_t)wgs), dim3(WR * WK * kWave), lds_bytes, st,
+                       static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C),
+                       ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
+    return (int)hipGetLastError();
+}
+
+// kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
+struct LaunchCfg { int kind, nt, rt, wr, wk; };
+
+inline size_t pow2_floor(size_t v)
+{
+    size_t p = 1;
+    while (p * 2 <= v) p *= 2;
+    return p;
+}
+
+// How many ways K should be cut (across workgroups via splitK and/or across the wavefronts of a tile workgroup) for
+// batches above 16: 128-row x (32|64)-column tiles give M/128 * column blocks workgroups of four wavefronts, and the
+// chip wants about four wavefronts per SIMD-less CU slot (4 * cus in total) before more parallelism stops paying.
+inline size_t tile_k_parallelism(size_t M, size_t N, int cus)
+{
+    size_t nt = N <= 32 ? 2 : 4, nblocks = (N + 16 * nt - 1) / (16 * nt), base = (M / 128) * nblocks;
+    size_t want = (size_t)(4.0 * cus / 1.5) / (base ? base : 1);
+    size_t p = pow2_floor(want ? want : 1);
+    return p > 16 ? 16 : p;
+}
+constexpr size_t kMaxAutoSplitK = 8;
+
+// Launch shape for a given splitK.
+//  N <= 16: stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M as long as
+//           M/(16*rt) workgroups still cover the compute units; wavefronts per workgroup follow the K blocks of one split
+//           and the register budget (16 wavefronts leave 128 VGPRs each).
+//  N > 16:  tile kernel, 128 rows x 32 or 64 columns, with the K parallelism that splitK leaves open given to the
+//           wavefronts of the workgroup (at most what its LDS holds).
+inline LaunchCfg pick_cfg(size_t M, size_t N, size_t K, int splitK, int cus)
+{
+    LaunchCfg c;
+    size_t    tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
+    if (N <= 16) {
+        c.kind = 0;
+        c.nt = 1;
+        c.wr = 1;
+        c.rt = 1;
+        while (c.rt < 4 && tiles % (2 * c.rt) == 0 && (tiles / (2 * c.rt)) * splitK >= (size_t)cus) c.rt *= 2;
+        int max_waves = c.rt <= 2 ? 16 : 8;
+        c.wk = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
+        if (c.wk > max_waves) c.wk = max_waves;
+        return c;
+    }
+    c.kind = 1;
+    c.nt = N <= 32 ? 2 : 4;
+    c.rt = 2;
+    c.wr = 4;
+    size_t open = tile_k_parallelism(M, N, cus) / (size_t)splitK;
+    if (open > per_split) open = per_split;
+    if (c.nt == 2 && open >= 4) {
+        c.rt = 1; // 64-row tiles: twice the workgroups, four K wavefronts each
+        c.wk = 4;
+    } else {
+        c.wk = open >= 2 ? 2 : 1;
+    }
     return c;
 }
 
 template <int XB>
-int launch_cfg(const StreamCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
+int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
                size_t K, int splitK)
 {
+    if (c.kind == 0) {
 #define FP6MI_CASE(NT, RT, WV) \
-    if (c.nt == NT && c.rt == RT && c.waves == WV) return launch_stream<XB, NT, RT, WV, false>(st, W, sc, B, C, ws, M, N, K, splitK);
-    FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
-    FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
-    FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
-    FP6MI_CASE(2, 1, 4) FP6MI_CASE(2, 1, 8)
-    FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
-    FP6MI_CASE(4, 1, 4) FP6MI_CASE(4, 1, 8)
-    FP6MI_CASE(4, 2, 4) FP6MI_CASE(4, 2, 8)
+    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV, false>(st, W, sc, B, C, ws, M, N, K, splitK);
+        FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
+        FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
+        FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
+        FP6MI_CASE(2, 1, 4) FP6MI_CASE(2, 1, 8)
+        FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
+        FP6MI_CASE(4, 1, 4) FP6MI_CASE(4, 1, 8)
+        FP6MI_CASE(4, 2, 4) FP6MI_CASE(4, 2, 8)
 #undef FP6MI_CASE
+    } else if (c.kind == 1) {
+#define FP6MI_CASE(NT, RT, WR, WK) \
+    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<XB, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
+        FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
+        FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
+        FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1)
+#undef FP6MI_CASE
+    }
     return FP6MI_ERR_SHAPE;
 }
 
 template <int XB>
 int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
-                  int splitK, const StreamCfg *forced)
+                  int splitK, const LaunchCfg *forced)
 {
-    StreamCfg c = forced ? *forced : pick_cfg(M, N, K, splitK, 256);
-    if ((M / 16) % c.rt) return FP6MI_ERR_SHAPE;
+    LaunchCfg c = forced ? *forced : pick_cfg(M, N, K, splitK, 256);
+    if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
     int rc = launch_cfg<XB>(c, st, W, sc, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
     if (splitK > 1) {
@@ -461,15 +718,26 @@ int fp6mi_relayout_ref_to_native(int E, int Mb, void *native, const void *ref, s
 
 size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK) { return splitK > 1 ? (size_t)splitK * M * N * sizeof(float) : 0; }
 
-// Cost model, in microseconds, of the stream kernel on a part with `num_cus` compute units: workgroups run in rounds of
-// one per CU, a workgroup streams its weights at what one CU sustains, the whole chip cannot beat HBM, and a split
-// costs a second launch plus writing and re-reading the FP32 partial sums.
+// Split-K choice.  Batches up to 16 (stream kernel): a cost model in microseconds on a part with `num_cus` compute
+// units -- workgroups run in rounds of one per CU, a workgroup streams its weights at what one CU sustains, the whole
+// chip cannot beat HBM, and a split costs a second launch plus writing and re-reading the FP32 partial sums; K is
+// already split inside the workgroup, so a split rarely pays.  Larger batches (tile kernel): as much of the wanted K
+// parallelism as keeps the FP32 partial-sum traffic (8 bytes per output per split) under half of the weight bytes.
 int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus)
 {
     if (M == 0 || N == 0 || K == 0 || num_cus <= 0) return 1;
+    size_t units = (K + 255) / 256;
+    if (N > 16) {
+        size_t p = tile_k_parallelism(M, N, num_cus);
+        size_t afford = (size_t)(0.5 * (double)K * 0.75 / (8.0 * (double)N));
+        size_t s = pow2_floor(afford ? afford : 1);
+        if (s > p) s = p;
+        if (s > kMaxAutoSplitK) s = kMaxAutoSplitK;
+        if (s > units) s = pow2_floor(units);
+        return (int)(s ? s : 1);
+    }
     const double cu_gbps = 60.0, hbm_gbps = 6000.0, launch_us = 3.0;
-    size_t       units = (K + 255) / 256, ntile = N <= 16 ? 16 : N <= 32 ? 32 : 64;
-    size_t       wgs = (M / 16 ? M / 16 : 1) * ((N + ntile - 1) / ntile);
+    size_t       wgs = M / 16 ? M / 16 : 1;
     double       best = 1e30;
     int          best_s = 1;
     for (int s = 1; s <= 64 && (size_t)s <= units; s++) {
@@ -507,11 +775,11 @@ int fp6mi_linear_native(int E, int Mb, void *stream, const void *W, const void *
 }
 
 int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
-                            float *ws, int splitK, int n_tiles, int row_tiles, int waves)
+                            float *ws, int splitK, int kind, int n_tiles, int row_tiles, int row_waves, int k_waves)
 {
     int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
     if (rc != FP6MI_OK) return rc;
-    StreamCfg   c = { n_tiles, row_tiles, waves };
+    LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
     return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, &c) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, &c);
 }

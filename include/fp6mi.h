@@ -80,11 +80,13 @@ int fp6mi_linear_native(int E, int Mbits, void *stream, const void *W_native, co
 
 /* Tuning hook: the same GEMM with the launch shape chosen by the caller instead of the built-in selection
  * (no counterpart in the reference, whose TilingConfig is picked inside fpx_linear_kernel, fp6_linear.cu:61-81).
- * n_tiles in {1,2,4} = 16-column batch tiles per workgroup, row_tiles in {1,2,4} = 16-row weight tiles per wavefront,
- * waves in {4,8,16} = wavefronts per workgroup.  Unsupported combinations return FP6MI_ERR_SHAPE. */
+ * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup),
+ * kind 1 = tile kernel (row_waves x k_waves wavefronts, activations staged in LDS);
+ * n_tiles = 16-column batch tiles per workgroup, row_tiles = 16-row weight tiles per wavefront.
+ * Combinations that are not compiled in, or that do not divide M, return FP6MI_ERR_SHAPE. */
 int fp6mi_linear_native_cfg(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
                             const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK,
-                            int n_tiles, int row_tiles, int waves);
+                            int kind, int n_tiles, int row_tiles, int row_waves, int k_waves);
 
 /* Device-side conversion reference layout -> native layout (both device pointers), run once per weight matrix. */
 int fp6mi_relayout_ref_to_native_gpu(int E, int Mbits, void *stream, void *native_dev, const void *packed_ref_dev,

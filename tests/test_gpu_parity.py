@@ -130,11 +130,19 @@ def test_split_k(E, M, splitK):
     check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "splitK=%d" % splitK)
 
 
-@pytest.mark.parametrize("cfg", [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 16), (1, 4, 8), (2, 1, 8), (2, 2, 4), (4, 1, 8), (4, 2, 8)])
-def test_every_launch_shape(cfg):
-    print("case launch shape", cfg, flush=True)
-    E, M = 3, 2
-    OC, IC, N = 512, 2304, 16 * cfg[0] - 3
+STREAM_SHAPES = [(0, 1, 1, 1, 4), (0, 1, 1, 1, 8), (0, 1, 1, 1, 16), (0, 1, 2, 1, 4), (0, 1, 2, 1, 8), (0, 1, 2, 1, 16), (0, 1, 4, 1, 4),
+                 (0, 1, 4, 1, 8), (0, 2, 1, 1, 4), (0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 2, 1, 8), (0, 4, 1, 1, 4), (0, 4, 1, 1, 8),
+                 (0, 4, 2, 1, 4), (0, 4, 2, 1, 8)]
+TILE_SHAPES = [(1, 2, 1, 4, 4), (1, 2, 2, 4, 4), (1, 2, 2, 4, 2), (1, 2, 2, 4, 1), (1, 2, 4, 4, 1), (1, 2, 4, 4, 2), (1, 4, 2, 4, 2),
+               (1, 4, 2, 4, 1), (1, 4, 4, 4, 1), (1, 4, 4, 2, 1), (1, 4, 4, 2, 2), (1, 8, 2, 4, 1), (1, 8, 2, 2, 1)]
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("cfg", STREAM_SHAPES + TILE_SHAPES)
+def test_every_launch_shape(E, M, cfg):
+    """Every compiled (kernel, tile) combination through the tuning hook: cfg = (kind, n_tiles, row_tiles, row_waves, k_waves)."""
+    print("case launch shape", E, M, cfg, flush=True)
+    OC, IC, N = 512, 2304, 16 * cfg[1] - 3
     raw, sc, x = synth.uniform_problem(500 + sum(cfg), OC, IC, N, E, M)
     native, scd, xd = upload(raw, sc, x, E, M)
     ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
@@ -147,8 +155,10 @@ def test_unsupported_launch_shape_is_rejected():
     native, scd, xd = upload(raw, sc, x, 3, 2)
     L = _lib.lib()
     out = torch.empty((4, 256), dtype=torch.float16, device=DEV)
-    rc = L.fp6mi_linear_native_cfg(3, 2, None, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), 256, 4, 256, None, 1, 3, 1, 8)
-    assert rc == -2
+    for bad in [(0, 3, 1, 1, 8), (0, 1, 1, 2, 8), (1, 2, 2, 4, 8), (2, 1, 1, 1, 4), (1, 4, 4, 4, 1)]:   # last: 256 rows per tile > M is fine, 4*4*16 = 256 divides; use M=256
+        rc = L.fp6mi_linear_native_cfg(3, 2, None, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), 256, 4, 256, None, 1, *bad)
+        assert rc == (-2 if bad != (1, 4, 4, 4, 1) else 0), bad
+    torch.cuda.synchronize()
 
 
 @pytest.mark.parametrize("E,M", FORMATS)

@@ -177,8 +177,12 @@ def test_reference_heuristic_is_kept_verbatim():
 
 
 def test_mi355x_heuristic_prefers_no_split_when_rows_fill_the_chip():
-    for (M, N, K) in [(4096, 8, 4096), (11008, 8, 4096), (8192, 32, 8192), (28672, 32, 8192), (8192, 512, 8192)]:
+    for (M, N, K) in [(4096, 8, 4096), (11008, 8, 4096), (8192, 16, 8192), (28672, 8, 8192), (8192, 512, 8192)]:
         assert fp6.heuristic_splitk_mi355x(M, N, K) == 1
+    # batches above 16 use 128-row tiles: K is cut until about four wavefronts per CU exist, partial-sum traffic permitting
+    assert fp6.heuristic_splitk_mi355x(8192, 32, 8192) == 8
+    assert fp6.heuristic_splitk_mi355x(28672, 32, 8192) == 2
+    assert fp6.heuristic_splitk_mi355x(8192, 64, 8192) == 4
     s = fp6.heuristic_splitk_mi355x(256, 8, 28672)      # 16 row tiles cannot occupy 256 CUs: splitting K pays
     assert 2 <= s <= 64
     assert fp6.heuristic_splitk_mi355x(256, 1, 1024) == 1  # too little work to pay for a second launch
