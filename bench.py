@@ -47,6 +47,13 @@ for _bs in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
     WORKLOADS["fp5_8192x8192_bs%d" % _bs] = (2, 2, 8192, 8192, _bs)
 HEADLINE = "fp6_4096x4096_bs8"
 
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
+# for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
+MEASURED_TRAFFIC_BYTES = {
+    "fp6_4096x4096_bs8": 13241840,
+    "fp6_28672x8192_bs32": 182294683,  # measured with the stream kernel; the tile kernel now serves this shape
+}
+
 
 def weight_bytes(E, M, OC, IC):
     return OC * IC * (1 + E + M) // 8
@@ -243,7 +250,7 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%s: FP%d_e%dm2 weights [%d,%d] x fp16 activations [%d,%d], weights rotating through %d distinct HBM buffers, splitK=%d"
                                % (args.workload, 1 + E + M, E, OC, IC, BS, IC, res["weight_buffers"], res["splitK"])},
-        "roofline": {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"], "traffic": None,
+        "roofline": {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "bytes_per_launch": res["weight_bytes"], "kernel_us": res["us_per_gemm"]},
         "detail": res,
     }

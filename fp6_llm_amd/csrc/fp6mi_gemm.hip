@@ -11,6 +11,9 @@
 // 2^14 exponent rebias of FP5) is applied once to the FP32 sums instead of to every weight.
 #include <hip/hip_runtime.h>
 
+#include <mutex>
+#include <unordered_map>
+
 #include "fp6mi_internal.h"
 
 namespace {
@@ -782,6 +785,69 @@ int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const vo
     LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
     return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, &c) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, &c);
+}
+
+// ---- drop-in entry on REFERENCE-layout weights: native twins are made on first sight of a weight pointer and kept ----
+namespace {
+struct Twin { void *native; int E, Mb; size_t M, K; int device; };
+std::mutex                              g_twin_mutex;
+std::unordered_map<const void *, Twin>  g_twins;
+} // namespace
+
+int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
+                 float *ws, int splitK)
+{
+    int rc = check_gemm_args(E, Mb, W_ref, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    int device = 0;
+    if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return (int)e;
+    void *native = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(g_twin_mutex);
+        auto it = g_twins.find(W_ref);
+        if (it != g_twins.end()) {
+            const Twin &t = it->second;
+            if (t.E == E && t.Mb == Mb && t.M == M && t.K == K && t.device == device) {
+                native = t.native;
+            } else { // the address now holds a different matrix
+                (void)hipFree(t.native);
+                g_twins.erase(it);
+            }
+        }
+        if (!native) {
+            size_t bytes = fp6mi::native_bytes(E, Mb, M, K);
+            if (hipError_t e = hipMalloc(&native, bytes); e != hipSuccess) return (int)e;
+            rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K); // same stream: ordered before the GEMM
+            if (rc != 0) {
+                (void)hipFree(native);
+                return rc;
+            }
+            g_twins[W_ref] = Twin{ native, E, Mb, M, K, device };
+        }
+    }
+    return fp6mi_linear_native(E, Mb, stream, native, sc, B, C, M, N, K, ws, splitK);
+}
+
+int fp6mi_twin_evict(const void *W_ref)
+{
+    std::lock_guard<std::mutex> lock(g_twin_mutex);
+    auto it = g_twins.find(W_ref);
+    if (it == g_twins.end()) return FP6MI_OK;
+    hipError_t e = hipFree(it->second.native); // hipFree waits for work that may still read the buffer
+    g_twins.erase(it);
+    return (int)e;
+}
+
+int fp6mi_twin_clear(void)
+{
+    std::lock_guard<std::mutex> lock(g_twin_mutex);
+    int rc = 0;
+    for (auto &kv : g_twins) {
+        hipError_t e = hipFree(kv.second.native);
+        if (e != hipSuccess) rc = (int)e;
+    }
+    g_twins.clear();
+    return rc;
 }
 
 int fp6mi_relayout_ref_to_native_gpu(int E, int Mb, void *stream, void *native, const void *ref, size_t M, size_t K)

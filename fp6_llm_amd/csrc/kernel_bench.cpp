@@ -8,10 +8,12 @@
 
 #include <cstdio>
 #include <cstdlib>
+#include <cmath>
 #include <random>
+#include <string>
 #include <vector>
 
-#include "../../include/fp6mi.h"
+#include "fp6_linear.h"
 
 #define HIP_OK(x)                                                                      \
     do {                                                                               \
@@ -22,8 +24,62 @@
         }                                                                              \
     } while (0)
 
+// `kernel_bench check E M OC IC BS SplitK`: the flow of the reference's C++ test (tests/cpp/kernel_test_fpx.cu:19-33,128-149)
+// through the reference-named C++ API: random raw bytes, dequantize on the CPU BEFORE prepacking in place, upload the
+// reference-layout buffer, run the GEMM, and print sum|err|/sum|ref| against a double-precision product of the
+// dequantized weights (tests/cpp/kernel_test.h:48-57).  Exit status 0 iff that ratio is below 2e-3.
+static int check_main(int argc, char **argv)
+{
+    if (argc < 8) { std::fprintf(stderr, "usage: %s check E M OC IC BS SplitK\n", argv[0]); return 1; }
+    int    E = std::atoi(argv[2]), Mb = std::atoi(argv[3]);
+    size_t OC = std::strtoull(argv[4], nullptr, 10), IC = std::strtoull(argv[5], nullptr, 10), BS = std::strtoull(argv[6], nullptr, 10);
+    int    splitK = std::atoi(argv[7]);
+    size_t wbytes = OC * IC * (1 + E + Mb) / 8;
+    std::vector<unsigned char> raw(wbytes);
+    std::mt19937               rng(7);
+    for (auto &b : raw) b = (unsigned char)(rng() & 255);
+    std::vector<fp6mi_half> sc(OC), x(BS * IC), wdq(OC * IC), out(BS * OC);
+    for (auto &v : sc) v = (fp6mi_half)((float)(rng() % 256 + 1) / 4096.0f);
+    for (auto &v : x) v = (fp6mi_half)(((int)(rng() % 5) - 2) * 0.1f - 0.1f);
+    if (int rc = dequant_matrix_fp_eXmY_to_fp16(E, Mb, wdq.data(), raw.data(), OC, IC, sc.data())) { std::fprintf(stderr, "dequant: %s\n", fp6mi_error_string(rc)); return 2; }
+    if (int rc = weight_matrix_prepacking_fp_eXmY(E, Mb, reinterpret_cast<int *>(raw.data()), reinterpret_cast<int *>(raw.data()), OC, IC)) {
+        std::fprintf(stderr, "prepack: %s\n", fp6mi_error_string(rc));
+        return 2;
+    }
+    void  *dW, *dS, *dX, *dC;
+    float *dWs = nullptr;
+    HIP_OK(hipMalloc(&dW, wbytes));
+    HIP_OK(hipMalloc(&dS, OC * 2));
+    HIP_OK(hipMalloc(&dX, BS * IC * 2));
+    HIP_OK(hipMalloc(&dC, BS * OC * 2));
+    HIP_OK(hipMemcpy(dW, raw.data(), wbytes, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dS, sc.data(), OC * 2, hipMemcpyHostToDevice));
+    HIP_OK(hipMemcpy(dX, x.data(), BS * IC * 2, hipMemcpyHostToDevice));
+    if (splitK > 1) HIP_OK(hipMalloc(reinterpret_cast<void **>(&dWs), fp6mi_workspace_bytes(OC, BS, splitK)));
+    for (int rep = 0; rep < 2; rep++) { // the second call reuses the native twin made by the first
+        int rc = fp_eXmY_linear_kernel(E, Mb, nullptr, dW, static_cast<fp6mi_half *>(dS), static_cast<fp6mi_half *>(dX), static_cast<fp6mi_half *>(dC), OC,
+                                       BS, IC, dWs, splitK);
+        if (rc) { std::fprintf(stderr, "fp_eXmY_linear_kernel: %s\n", fp6mi_error_string(rc)); return 2; }
+    }
+    HIP_OK(hipDeviceSynchronize());
+    HIP_OK(hipMemcpy(out.data(), dC, BS * OC * 2, hipMemcpyDeviceToHost));
+    long double err = 0, ref = 0;
+    for (size_t n = 0; n < BS; n++)
+        for (size_t m = 0; m < OC; m++) {
+            double acc = 0;
+            for (size_t k = 0; k < IC; k++) acc += (double)wdq[m * IC + k] * (double)x[n * IC + k];
+            err += std::fabs((double)out[n * OC + m] - acc);
+            ref += std::fabs(acc);
+        }
+    double ratio = (double)(err / ref);
+    std::printf("check E%dM%d OC=%zu IC=%zu BS=%zu splitK=%d: sum|err|/sum|ref| = %.3e\n", E, Mb, OC, IC, BS, splitK, ratio);
+    if (int rc = fp6mi_twin_clear()) { std::fprintf(stderr, "twin_clear: %s\n", fp6mi_error_string(rc)); return 2; }
+    return ratio < 2e-3 ? 0 : 3;
+}
+
 int main(int argc, char **argv)
 {
+    if (argc > 1 && std::string(argv[1]) == "check") return check_main(argc, argv);
     if (argc < 7) {
         std::fprintf(stderr, "usage: %s E M OC IC BS SplitK [iters] [warmup] [pool_MiB]\n", argv[0]);
         return 1;

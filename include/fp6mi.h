@@ -78,6 +78,17 @@ size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK);
 int fp6mi_linear_native(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
                         const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK);
 
+/* Drop-in for fp_eXmY_linear_kernel / fp6_linear_kernel (fp6_llm/csrc/fp6_linear.cuh:8-32): W is the REFERENCE
+ * prepacked layout on the device, exactly what a caller of the reference already holds.  On the first call with a
+ * given W pointer the library allocates a native-layout twin (hipMalloc) and fills it with one relayout kernel on
+ * `stream`; later calls with the same (pointer, format, M, K) reuse it.  The twin is keyed by ADDRESS: if the caller
+ * overwrites or frees-and-reuses the weight buffer it must call fp6mi_twin_evict(W) (or fp6mi_twin_clear()) first.
+ * Callers that cannot tolerate the hidden allocation convert explicitly and use fp6mi_linear_native. */
+int fp6mi_linear(int E, int Mbits, void *stream, const void *W_ref, const void *scales_f16, const void *B_f16,
+                 void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK);
+int fp6mi_twin_evict(const void *W_ref);
+int fp6mi_twin_clear(void);
+
 /* Tuning hook: the same GEMM with the launch shape chosen by the caller instead of the built-in selection
  * (no counterpart in the reference, whose TilingConfig is picked inside fpx_linear_kernel, fp6_linear.cu:61-81).
  * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup),

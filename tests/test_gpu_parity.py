@@ -208,6 +208,47 @@ def test_reference_named_api_both_argument_orders(E, M):
     assert (y4 == 0).all()
 
 
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_c_abi_drop_in_on_reference_layout(E, M):
+    """fp6mi_linear takes the reference's prepacked bytes as they are; its native twin is keyed by address."""
+    L = _lib.lib()
+    OC, IC, N = 256, 1024, 12
+    raw, sc, x = synth.uniform_problem(700, OC, IC, N, E, M)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    out = torch.empty((N, OC), dtype=torch.float16, device=DEV)
+    ws = torch.empty(3 * N * OC, dtype=torch.float32, device=DEV)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    for splitK in (1, 3, 1):
+        rc = L.fp6mi_linear(E, M, torch.cuda.current_stream().cuda_stream, packed.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(),
+                            OC, N, IC, ws.data_ptr(), splitK)
+        assert rc == 0, L.fp6mi_error_string(rc)
+        torch.cuda.synchronize()
+        check_close(out.cpu().numpy(), ref, "fp6mi_linear splitK=%d" % splitK)
+    # same address, new contents: the caller evicts the twin
+    raw2, _, _ = synth.uniform_problem(701, OC, IC, N, E, M)
+    packed.copy_(fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw2)))
+    assert L.fp6mi_twin_evict(packed.data_ptr()) == 0
+    rc = L.fp6mi_linear(E, M, torch.cuda.current_stream().cuda_stream, packed.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(),
+                        OC, N, IC, None, 1)
+    assert rc == 0
+    torch.cuda.synchronize()
+    check_close(out.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw2, sc, E, M), x), "after evict")
+    assert L.fp6mi_twin_clear() == 0
+
+
+def test_cpp_api_driver():
+    """The reference-named C++ API (fp6_llm_amd/csrc/fp6_linear.h) through the command-line driver, in the order the
+    reference's C++ test uses it: dequantize, prepack in place, upload, GEMM."""
+    import os
+    import subprocess
+    exe = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fp6_llm_amd", "kernel_bench")
+    assert os.path.exists(exe), "kernel_bench is built by __graft_entry__.build()"
+    for args in (["3", "2", "256", "512", "8", "1"], ["2", "2", "512", "1024", "33", "2"]):
+        res = subprocess.run([exe, "check"] + args, capture_output=True, text=True, timeout=120)
+        assert res.returncode == 0, res.stdout + res.stderr
+
+
 # ------------------------------------------------------------------------------------------------ benchmark configs
 def _bench_case(E, M, OC, IC, BS, seed, gaussian, act_sigma=1.0, splitKs=(None,)):
     print("case bench config", E, M, OC, IC, BS, flush=True)
