@@ -115,25 +115,40 @@ template <int XB, int NT, int RT> struct Stage {
 
 template <int XB, int NT, int RT>
 __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
-                                           const half_t *const (&xrow)[NT], const bool (&xok)[NT], int q, uint32_t K)
+                                           const half_t *const (&xrow)[NT], int q, uint32_t K)
 {
+#ifndef FP6MI_EXP_XFIRST
 #pragma unroll
     for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
+#endif
 #ifndef FP6MI_EXP_NOX
+    // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
+    // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
+    // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
+    if ((u + 1) * 256 <= K) { // uniform: whole block inside K, one base address and immediate offsets
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        uint32_t k = u * 256 + 32 * s;
+        for (int s = 0; s < 8; s++)
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            v8h z = { 0, 0, 0, 0, 0, 0, 0, 0 };
-            st.x[s][t] = (xok[t] && k + 8 * q < K) ? *reinterpret_cast<const v8h *>(xrow[t] + k) : z;
+            for (int t = 0; t < NT; t++) st.x[s][t] = *reinterpret_cast<const v8h *>(xrow[t] + u * 256 + 32 * s);
+    } else {
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            uint32_t k = u * 256 + 32 * s;
+            if (k + 8 * q >= K) k = 0;
+#pragma unroll
+            for (int t = 0; t < NT; t++) st.x[s][t] = *reinterpret_cast<const v8h *>(xrow[t] + k);
         }
     }
+    __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
 #else
 #pragma unroll
     for (int s = 0; s < 8; s++)
 #pragma unroll
         for (int t = 0; t < NT; t++) { v8h o = { 1, 1, 1, 1, 1, 1, 1, 1 }; st.x[s][t] = o; }
+#endif
+#ifdef FP6MI_EXP_XFIRST
+#pragma unroll
+    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
 #endif
 }
 
@@ -177,12 +192,20 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
 
     const half_t *xrow[NT];
-    bool          xok[NT];
 #pragma unroll
     for (int t = 0; t < NT; t++) {
         uint32_t n = nbase + 16 * t + col;
-        xok[t]     = n < N;
-        xrow[t]    = X + (size_t)(xok[t] ? n : 0) * K + 8 * q;
+        xrow[t]    = X + (size_t)(n < N ? n : N - 1) * K + 8 * q;
+    }
+
+    // The epilogue gives thread e the output (row tile e/(256*NT), column tile, batch column, row e%16); its row scale is
+    // fetched now so that no global load sits on the tail of the kernel.
+    constexpr int kOutPerThread = (RT * NT * 256 + WAVES * kWave - 1) / (WAVES * kWave);
+    half_t        my_scale[kOutPerThread]; // kept as loaded: converting here would wait for the load before the weight loads issue
+#pragma unroll
+    for (int j = 0; j < kOutPerThread; j++) {
+        int e = threadIdx.x + j * WAVES * kWave;
+        my_scale[j] = scales[(R0 + (e < RT * NT * 256 ? (e >> 8) / NT : 0)) * 16 + (e & 15)];
     }
 
     // workgroups that share an L2 (ids congruent mod 8) start on different K blocks, so that the chip does not ask
@@ -191,12 +214,12 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     if (PF) {
         if (u < u1) {
             Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, xok, q, K);
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K);
             for (;;) {
                 uint32_t   un = u + WAVES;
                 const bool more = un < u1;
                 Stage<XB, NT, RT> nxt;
-                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, xok, q, K);
+                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, q, K);
                 consume_stage<XB, NT, RT>(cur, acc);
                 if (!more) break;
                 cur = nxt;
@@ -206,7 +229,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     } else {
         for (; u < u1; u += WAVES) {
             Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, xok, q, K);
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K);
             consume_stage<XB, NT, RT>(cur, acc);
         }
     }
@@ -218,7 +241,10 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[wave][r * NT + t][lane * 4]) = acc[r][t];
     __syncthreads();
 
-    for (int e = threadIdx.x; e < RT * NT * 256; e += WAVES * kWave) {
+#pragma unroll
+    for (int j = 0; j < kOutPerThread; j++) {
+        const int e = threadIdx.x + j * WAVES * kWave;
+        if (e >= RT * NT * 256) break;
         int   rt = e >> 8, i8 = e & 255, n = i8 >> 4, mm = i8 & 15;
         int   r = rt / NT, t = rt % NT;
         int   idx = (((mm >> 2) * 16 + n) << 2) | (mm & 3);
@@ -227,7 +253,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         for (int w = 0; w < WAVES; w++) sum += red[w][rt][idx];
         uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
         if (ng < N) {
-            float v = sum * ((float)scales[mg] * Fmt<XB>::post_scale);
+            float v = sum * ((float)my_scale[j] * Fmt<XB>::post_scale);
             if (splitK == 1)
                 C[(size_t)ng * M + mg] = (half_t)v;
             else
@@ -311,6 +337,13 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     WFrag<XB> wcur[RT], wnxt[RT];
     v4u       xr[kPerThread];
 
+    // row scales of this lane's outputs (rows 4q..4q+3 of each of its row tiles), fetched before the main loop so that no
+    // global load sits on the tail of the kernel
+    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+    v4h sc4[RT];
+#pragma unroll
+    for (int r = 0; r < RT; r++) sc4[r] = *reinterpret_cast<const v4h *>(scales + (R0 + r) * 16 + 4 * q);
+
     auto load_w = [&](WFrag<XB>(&dst)[RT], uint32_t c0) {
         const uint32_t u = c0 + wk;
         if (u < u1) {
@@ -322,11 +355,13 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
         for (int j = 0; j < kPerThread; j++) {
             const uint32_t p = tid + NTHREADS * j;
-            v4u            z = { 0, 0, 0, 0 };
-            xr[j]            = z;
             if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
-                const uint32_t k = (c0 + p / (TN * 32)) * 256 + (p & 31) * 8, n = nbase + (p >> 5) % TN;
-                if (n < N && k < K && c0 + p / (TN * 32) < u1) xr[j] = *reinterpret_cast<const v4u *>(X + (size_t)n * K + k);
+                // no zero fill: columns beyond N read the last real row (their outputs are never stored), positions beyond
+                // K or beyond the split read position 0 of the row (zero weights there, or a wavefront that does not compute)
+                uint32_t       k = (c0 + p / (TN * 32)) * 256 + (p & 31) * 8;
+                const uint32_t n = nbase + (p >> 5) % TN;
+                if (k >= K || c0 + p / (TN * 32) >= u1) k = 0;
+                xr[j] = *reinterpret_cast<const v4u *>(X + (size_t)(n < N ? n : N - 1) * K + k);
             }
         }
     };
@@ -401,15 +436,13 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
         for (int r = 0; r < RT; r++) {
             const uint32_t mg = (R0 + r) * 16 + 4 * q;
-            typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-            const v4h sc4 = *reinterpret_cast<const v4h *>(scales + mg);
 #pragma unroll
             for (int t = 0; t < NT; t++) {
                 const uint32_t ng = nbase + 16 * t + col;
                 if (ng < N) {
                     v4f v;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[i] * Fmt<XB>::post_scale);
+                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<XB>::post_scale);
                     if (splitK == 1) {
                         v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
                         *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
