@@ -619,6 +619,9 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
 }
 
 // kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
+#ifndef FP6MI_PF
+#define FP6MI_PF false
+#endif
 struct LaunchCfg { int kind, nt, rt, wr, wk; };
 
 inline size_t pow2_floor(size_t v)
@@ -641,12 +644,11 @@ inline size_t tile_k_parallelism(size_t M, size_t N, int cus)
 constexpr size_t kMaxAutoSplitK = 8;
 
 // Launch shape for a given splitK.
-//  N <= 16: stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M as long as
-//           M/(16*rt) workgroups still cover the compute units; wavefronts per workgroup follow the K blocks of one split
-//           and the register budget (16 wavefronts leave 128 VGPRs each).
+//  N <= 16: stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M; wavefronts
+//           per workgroup follow the K blocks of one split and the register budget (16 wavefronts leave 128 VGPRs each).
 //  N > 16:  tile kernel, 128 rows x 32 or 64 columns, with the K parallelism that splitK leaves open given to the
 //           wavefronts of the workgroup (at most what its LDS holds).
-inline LaunchCfg pick_cfg(size_t M, size_t N, size_t K, int splitK, int cus)
+inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, int cus)
 {
     LaunchCfg c;
     size_t    tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
@@ -654,11 +656,19 @@ inline LaunchCfg pick_cfg(size_t M, size_t N, size_t K, int splitK, int cus)
         c.kind = 0;
         c.nt = 1;
         c.wr = 1;
-        c.rt = 1;
-        while (c.rt < 4 && tiles % (2 * c.rt) == 0 && (tiles / (2 * c.rt)) * splitK >= (size_t)cus) c.rt *= 2;
-        int max_waves = c.rt <= 2 ? 16 : 8;
-        c.wk = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
-        if (c.wk > max_waves) c.wk = max_waves;
+        // measured on MI355X: sharing the activation registers among four row tiles wins as soon as M/64 workgroups of four
+        // wavefronts cover about 60 % of the CUs; two row tiles need a full set of workgroups; otherwise one row tile
+        // per workgroup with as many wavefronts as there are K blocks to hand out.
+        if (tiles % 4 == 0 && (tiles / 4) * splitK * 100 >= (size_t)cus * 60) {
+            c.rt = 4;
+            c.wk = 4;
+        } else if (tiles % 2 == 0 && (tiles / 2) * splitK >= (size_t)cus) {
+            c.rt = 2;
+            c.wk = per_split > 8 ? (xbits == 5 ? 8 : 16) : per_split > 4 ? 8 : 4;
+        } else {
+            c.rt = 1;
+            c.wk = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
+        }
         return c;
     }
     c.kind = 1;
@@ -682,7 +692,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
 {
     if (c.kind == 0) {
 #define FP6MI_CASE(NT, RT, WV) \
-    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV, false>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV, FP6MI_PF>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
         FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
@@ -706,7 +716,7 @@ template <int XB>
 int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
                   int splitK, const LaunchCfg *forced)
 {
-    LaunchCfg c = forced ? *forced : pick_cfg(M, N, K, splitK, 256);
+    LaunchCfg c = forced ? *forced : pick_cfg(XB, M, N, K, splitK, 256);
     if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
     int rc = launch_cfg<XB>(c, st, W, sc, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
