@@ -1,0 +1,105 @@
+"""Caller-side conveniences around the linear-layer path: a torch module that owns native-layout weights, and a small
+on-disk container for them.  (The reference leaves both to the framework that embeds it -- DeepSpeed, README.md:19.)"""
+import json
+import struct
+
+import numpy as np
+import torch
+
+from . import quant
+from . import (MI355X_CUS, heuristic_splitk_mi355x, linear_forward_native, native_bytes, to_native,
+               weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu)
+
+_MAGIC = b"FP6MI\x00\x01\x00"   # name, NUL, layout version 1, reserved
+
+
+class FPxLinear(torch.nn.Module):
+    """y = x @ dequant(W)^T (+ bias) with W held in the native gfx950 layout.  Weights are buffers, not parameters:
+    the layer is inference-only, like the kernels."""
+
+    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None):
+        super().__init__()
+        if out_features % 256 or in_features % 64:
+            raise ValueError("FPxLinear needs out_features %% 256 == 0 and in_features %% 64 == 0")
+        self.in_features, self.out_features = in_features, out_features
+        self.exponent, self.mantissa = exponent, mantissa
+        self.split_k = split_k
+        self.register_buffer("weight_native", torch.zeros(native_bytes(exponent, mantissa, out_features, in_features) // 4, dtype=torch.int32))
+        self.register_buffer("scales", torch.ones(out_features, dtype=torch.float16))
+        self.register_buffer("bias", bias)
+
+    @classmethod
+    def from_raw(cls, raw_int32, scales, exponent=3, mantissa=2, bias=None, split_k=None):
+        """raw_int32: the reference's raw weight tensor [OC, IC/32*x] (CPU); scales: float16 [OC]."""
+        x = 1 + exponent + mantissa
+        OC, IC = raw_int32.shape[0], raw_int32.shape[1] * 32 // x
+        m = cls(IC, OC, exponent, mantissa, bias, split_k)
+        m.weight_native.copy_(weight_prepacking_native_cpu(exponent, mantissa, raw_int32))
+        m.scales.copy_(scales)
+        return m
+
+    @classmethod
+    def from_prepacked(cls, packed_int32, scales, exponent=3, mantissa=2, bias=None, split_k=None):
+        """packed_int32: output of weight_prepacking*_cpu (the reference layout), on CPU or GPU."""
+        x = 1 + exponent + mantissa
+        OC, IC = packed_int32.shape[0], packed_int32.shape[1] * 32 // x
+        m = cls(IC, OC, exponent, mantissa, bias, split_k).to(packed_int32.device)
+        m.weight_native.copy_(to_native(packed_int32, exponent, mantissa))
+        m.scales.copy_(scales.to(packed_int32.device))
+        return m
+
+    @classmethod
+    def from_float(cls, weight, exponent=3, mantissa=2, bias=None, split_k=None):
+        """Quantizes a float [OC, IC] weight row-wise (round to nearest even, absmax scales) and packs it."""
+        codes, scales = quant.quantize_rowwise(weight.detach().float().cpu().numpy(), exponent, mantissa)
+        raw = torch.from_numpy(quant.pack_raw(codes, exponent, mantissa))
+        return cls.from_raw(raw, torch.from_numpy(scales), exponent, mantissa, bias, split_k)
+
+    def forward(self, x):
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, self.in_features)
+        if x2.dtype != torch.float16:
+            x2 = x2.half()
+        sk = self.split_k or heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS)
+        y = linear_forward_native(self.exponent, self.mantissa, x2, self.weight_native, self.scales, self.out_features, sk)
+        if self.bias is not None:
+            y = y + self.bias
+        return y.reshape(*lead, self.out_features)
+
+    def extra_repr(self):
+        return "in_features=%d, out_features=%d, format=e%dm%d" % (self.in_features, self.out_features, self.exponent, self.mantissa)
+
+
+def save_native(path, native_int32, scales, exponent, mantissa, out_features, in_features):
+    """One weight matrix in the native layout: magic, little-endian uint32 header length, JSON header, native bytes, fp16 scales."""
+    nat = native_int32.detach().cpu().contiguous().numpy()
+    sc = scales.detach().cpu().contiguous().numpy().astype(np.float16)
+    if nat.nbytes != native_bytes(exponent, mantissa, out_features, in_features) or sc.shape != (out_features,):
+        raise ValueError("buffers do not match the stated shape")
+    header = json.dumps({"exponent": exponent, "mantissa": mantissa, "out_features": out_features, "in_features": in_features,
+                         "layout": "native-v1", "native_bytes": int(nat.nbytes)}).encode()
+    with open(path, "wb") as f:
+        f.write(_MAGIC)
+        f.write(struct.pack("<I", len(header)))
+        f.write(header)
+        f.write(nat.tobytes())
+        f.write(sc.tobytes())
+
+
+def load_native(path):
+    """Returns (native int32 tensor, float16 scales, header dict).  Plain binary parsing; nothing in the file is executed."""
+    with open(path, "rb") as f:
+        if f.read(len(_MAGIC)) != _MAGIC:
+            raise ValueError("%s is not a native FPx weight file (or has another layout version)" % path)
+        (hlen,) = struct.unpack("<I", f.read(4))
+        if hlen > 1 << 16:
+            raise ValueError("implausible header length")
+        hdr = json.loads(f.read(hlen).decode())
+        want = native_bytes(hdr["exponent"], hdr["mantissa"], hdr["out_features"], hdr["in_features"])
+        if hdr.get("layout") != "native-v1" or hdr.get("native_bytes") != want:
+            raise ValueError("header does not describe a native-v1 weight of that shape")
+        nat = np.frombuffer(f.read(want), dtype=np.int32)
+        sc = np.frombuffer(f.read(2 * hdr["out_features"]), dtype=np.float16)
+        if nat.nbytes != want or sc.size != hdr["out_features"]:
+            raise ValueError("file is truncated")
+    return torch.from_numpy(nat.copy()), torch.from_numpy(sc.copy()), hdr

@@ -249,6 +249,50 @@ def test_cpp_api_driver():
         assert res.returncode == 0, res.stdout + res.stderr
 
 
+def test_graph_capture_replays_match_eager():
+    """Both kernels, with and without split-K, captured into a HIP graph and replayed with new activations between
+    replays; every replay must equal the eager result bit for bit (the library records no memset nodes)."""
+    E, M = 3, 2
+    OC, IC = 512, 2048
+    raw, sc, _ = synth.uniform_problem(800, OC, IC, 1, E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd = torch.from_numpy(sc).to(DEV)
+    for N, splitK in ((8, 1), (8, 3), (40, 1), (40, 4)):
+        x = torch.zeros((N, IC), dtype=torch.float16, device=DEV)
+        out = torch.empty((N, OC), dtype=torch.float16, device=DEV)
+        ws = torch.empty(splitK * N * OC, dtype=torch.float32, device=DEV)
+        s = torch.cuda.Stream()
+        with torch.cuda.stream(s):
+            fp6.linear_forward_native(E, M, x, native, scd, OC, splitK, out=out, workspace=ws)
+            torch.cuda.synchronize()
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=s):
+                fp6.linear_forward_native(E, M, x, native, scd, OC, splitK, out=out, workspace=ws)
+        for rep in range(3):
+            xin = torch.from_numpy(synth.activations(810 + rep, N, IC)).to(DEV)
+            eager = fp6.linear_forward_native(E, M, xin, native, scd, OC, splitK)
+            torch.cuda.synchronize()
+            x.copy_(xin)
+            g.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, eager), (N, splitK, rep)
+
+
+def test_module_forward():
+    from fp6_llm_amd import module
+    w = torch.from_numpy(synth.normal(31, (512, 1024))).float()
+    bias = torch.from_numpy(synth.normal(32, (512,))).half()
+    for (E, M) in FORMATS:
+        layer = module.FPxLinear.from_float(w, E, M, bias=bias).to(DEV)
+        x = torch.from_numpy(synth.activations(33, 2 * 5, 1024)).reshape(2, 5, 1024).to(DEV)
+        y = layer(x)
+        assert y.shape == (2, 5, 512)
+        codes, scales = quant.quantize_rowwise(w.numpy(), E, M)
+        wdq = oracle.dequant(quant.pack_raw(codes, E, M), scales, E, M)
+        ref = oracle.gemm_f64(wdq, x.reshape(10, 1024).cpu().numpy()) + bias.double().numpy()
+        check_close(y.reshape(10, 512).cpu().numpy(), ref, "module e%dm%d" % (E, M))
+
+
 # ------------------------------------------------------------------------------------------------ benchmark configs
 def _bench_case(E, M, OC, IC, BS, seed, gaussian, act_sigma=1.0, splitKs=(None,)):
     print("case bench config", E, M, OC, IC, BS, flush=True)

@@ -211,3 +211,36 @@ def test_quantizer(E, M):
     assert np.abs(deq - w).max() <= np.abs(w).max() / mags[-1] * np.diff(mags).max() * 0.51
     raw = quant.pack_raw(codes, E, M)
     assert (quant.unpack_raw(raw, E, M) == codes).all() and (oracle.unpack_codes(raw, E, M) == codes).all()
+
+
+def test_native_weight_file_round_trip(tmp_path):
+    from fp6_llm_amd import module
+    raw, sc = _problem(21, 256, 320, 2, 2)
+    nat = fp6.weight_prepacking_native_cpu(2, 2, torch.from_numpy(raw))
+    path = str(tmp_path / "w.fp6mi")
+    module.save_native(path, nat, torch.from_numpy(sc), 2, 2, 256, 320)
+    nat2, sc2, hdr = module.load_native(path)
+    assert torch.equal(nat, nat2) and (sc2.numpy() == sc).all() and hdr["in_features"] == 320 and hdr["exponent"] == 2
+    with open(path, "r+b") as f:
+        f.truncate(4000)
+    with pytest.raises(ValueError):
+        module.load_native(path)
+    with open(path, "wb") as f:
+        f.write(b"not a weight file")
+    with pytest.raises(ValueError):
+        module.load_native(path)
+
+
+def test_module_construction_routes_agree():
+    from fp6_llm_amd import module
+    raw, sc = _problem(22, 256, 128, 3, 2)
+    t, s = torch.from_numpy(raw), torch.from_numpy(sc)
+    a = module.FPxLinear.from_raw(t, s)
+    b = module.FPxLinear.from_prepacked(fp6.weight_prepacking_cpu(t), s)
+    assert torch.equal(a.weight_native, b.weight_native) and torch.equal(a.scales, b.scales)
+    w = torch.from_numpy(synth.normal(3, (256, 128))).float()
+    c = module.FPxLinear.from_float(w)
+    codes, scales = quant.quantize_rowwise(w.numpy(), 3, 2)
+    assert torch.equal(c.weight_native, fp6.weight_prepacking_native_cpu(3, 2, torch.from_numpy(quant.pack_raw(codes, 3, 2))))
+    with pytest.raises(ValueError):
+        module.FPxLinear(100, 256)
