@@ -346,12 +346,22 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 
     auto load_w = [&](WFrag<XB>(&dst)[RT], uint32_t c0) {
         const uint32_t u = c0 + wk;
+#ifdef FP6MI_EXP_NOWT
+        if (u == u0 + wk) {
+#else
         if (u < u1) {
+#endif
 #pragma unroll
             for (int r = 0; r < RT; r++) dst[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
         }
     };
     auto load_x = [&](uint32_t c0) {
+#ifdef FP6MI_EXP_NOXT
+        return;
+#endif
+#ifdef FP6MI_EXP_NOXLOAD
+        if (c0 != u0) return;
+#endif
 #pragma unroll
         for (int j = 0; j < kPerThread; j++) {
             const uint32_t p = tid + NTHREADS * j;
@@ -366,6 +376,9 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         }
     };
     auto store_x = [&](int buf) {
+#ifdef FP6MI_EXP_NOXT
+        return;
+#endif
 #pragma unroll
         for (int j = 0; j < kPerThread; j++) {
             const uint32_t p = tid + NTHREADS * j;
@@ -397,7 +410,11 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
                     for (int s = 0; s < 4; s++) {
                         v8h b[NT];
 #pragma unroll
+#ifdef FP6MI_EXP_NOLDS
+                        for (int t = 0; t < NT; t++) { v8h o = { 1, 1, 1, 1, 1, 1, 1, 1 }; b[t] = o * (half_t)(float)(t + s + lane); }
+#else
                         for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xs + t * 16 * kXsRowBytes + (4 * h + s) * 64);
+#endif
 #pragma unroll
                         for (int r = 0; r < RT; r++)
 #pragma unroll
@@ -677,9 +694,13 @@ inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, i
     c.wr = 4;
     size_t open = tile_k_parallelism(M, N, cus) / (size_t)splitK;
     if (open > per_split) open = per_split;
+    size_t nblocks = (N + 16 * c.nt - 1) / (16 * c.nt);
     if (c.nt == 2 && open >= 4) {
         c.rt = 1; // 64-row tiles: twice the workgroups, four K wavefronts each
         c.wk = 4;
+    } else if (c.nt == 4 && open < 2 && M % 256 == 0 && (M / 256) * nblocks * splitK >= (size_t)cus) {
+        c.wr = 8; // enough 256-row tiles for every CU: the staged activation chunk then serves twice the rows
+        c.wk = 1;
     } else {
         c.wk = open >= 2 ? 2 : 1;
     }
@@ -706,7 +727,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
     if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<XB, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
         FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
-        FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1)
+        FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1)
 #undef FP6MI_CASE
     }
     return FP6MI_ERR_SHAPE;

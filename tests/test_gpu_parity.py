@@ -134,7 +134,8 @@ STREAM_SHAPES = [(0, 1, 1, 1, 4), (0, 1, 1, 1, 8), (0, 1, 1, 1, 16), (0, 1, 2, 1
                  (0, 1, 4, 1, 8), (0, 2, 1, 1, 4), (0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 2, 1, 8), (0, 4, 1, 1, 4), (0, 4, 1, 1, 8),
                  (0, 4, 2, 1, 4), (0, 4, 2, 1, 8)]
 TILE_SHAPES = [(1, 2, 1, 4, 4), (1, 2, 2, 4, 4), (1, 2, 2, 4, 2), (1, 2, 2, 4, 1), (1, 2, 4, 4, 1), (1, 2, 4, 4, 2), (1, 4, 2, 4, 2),
-               (1, 4, 2, 4, 1), (1, 4, 4, 4, 1), (1, 4, 4, 2, 1), (1, 4, 4, 2, 2), (1, 8, 2, 4, 1), (1, 8, 2, 2, 1)]
+               (1, 4, 2, 4, 1), (1, 4, 4, 4, 1), (1, 4, 4, 2, 1), (1, 4, 4, 2, 2), (1, 8, 2, 4, 1), (1, 8, 2, 2, 1), (1, 4, 2, 8, 1), (1, 4, 2, 8, 2), (1, 2, 2, 8, 1),
+               (1, 2, 2, 8, 2), (1, 8, 2, 8, 1), (1, 4, 1, 8, 2), (1, 4, 1, 8, 1)]
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
