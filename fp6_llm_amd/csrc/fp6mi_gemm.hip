@@ -355,23 +355,35 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
             for (int r = 0; r < RT; r++) dst[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
         }
     };
+    // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
+    // batch column (p/32) % TN, halfs 8*(p%32)..+7).  Row pointers and LDS offsets are fixed for the whole kernel.
+    // There is no zero fill: columns beyond N read the last real row (their outputs are never stored); positions beyond K or
+    // beyond the split read position 0 of the row (zero weights there, or a wavefront that does not compute).
+    const half_t *xrow[kPerThread];
+    uint32_t      xlds[kPerThread];
+#pragma unroll
+    for (int j = 0; j < kPerThread; j++) {
+        const uint32_t p = tid + NTHREADS * j, n = nbase + (p >> 5) % TN;
+        xrow[j] = X + (size_t)(n < N ? n : N - 1) * K + (p & 31) * 8 + (size_t)(p / (TN * 32)) * 256;
+        xlds[j] = (p >> 5) * kXsRowBytes + (p & 31) * 16;
+    }
     auto load_x = [&](uint32_t c0) {
 #ifdef FP6MI_EXP_NOXT
         return;
 #endif
-#ifdef FP6MI_EXP_NOXLOAD
-        if (c0 != u0) return;
-#endif
+        if ((c0 + WK) * 256 <= K && c0 + WK <= u1) { // uniform: the whole chunk lies inside K and inside the split
 #pragma unroll
-        for (int j = 0; j < kPerThread; j++) {
-            const uint32_t p = tid + NTHREADS * j;
-            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
-                // no zero fill: columns beyond N read the last real row (their outputs are never stored), positions beyond
-                // K or beyond the split read position 0 of the row (zero weights there, or a wavefront that does not compute)
-                uint32_t       k = (c0 + p / (TN * 32)) * 256 + (p & 31) * 8;
-                const uint32_t n = nbase + (p >> 5) % TN;
-                if (k >= K || c0 + p / (TN * 32) >= u1) k = 0;
-                xr[j] = *reinterpret_cast<const v4u *>(X + (size_t)(n < N ? n : N - 1) * K + k);
+            for (int j = 0; j < kPerThread; j++)
+                if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kPerThread; j++) {
+                const uint32_t p = tid + NTHREADS * j;
+                if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
+                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
+                    const bool     ok = k < K && u < u1;
+                    xr[j] = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                }
             }
         }
     };
@@ -380,11 +392,8 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         return;
 #endif
 #pragma unroll
-        for (int j = 0; j < kPerThread; j++) {
-            const uint32_t p = tid + NTHREADS * j;
-            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces)
-                *reinterpret_cast<v4u *>(lds + buf * kBufBytes + (p >> 5) * kXsRowBytes + (p & 31) * 16) = xr[j];
-        }
+        for (int j = 0; j < kPerThread; j++)
+            if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) *reinterpret_cast<v4u *>(lds + buf * kBufBytes + xlds[j]) = xr[j];
     };
 
     if (u0 < u1) {
@@ -401,11 +410,14 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
             }
             if (c0 + wk < u1) {
                 const uint8_t *xs = lds + buf * kBufBytes + (wk * TN + col) * kXsRowBytes + q * 16;
+                v8h            a0[RT][4], a1[RT][4];
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half(wcur[r], 0, a0[r]);
+                // second half converted ahead of the first half's MFMAs: the VALU work then runs under the matrix pipe
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half(wcur[r], 1, a1[r]);
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
-                    v8h a[RT][4];
-#pragma unroll
-                    for (int r = 0; r < RT; r++) convert_half(wcur[r], h, a[r]);
 #pragma unroll
                     for (int s = 0; s < 4; s++) {
                         v8h b[NT];
@@ -418,7 +430,8 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
                         for (int r = 0; r < RT; r++)
 #pragma unroll
-                            for (int t = 0; t < NT; t++) acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[r][s], b[t], acc[r][t], 0, 0, 0);
+                            for (int t = 0; t < NT; t++)
+                                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h == 0 ? a0[r][s] : a1[r][s], b[t], acc[r][t], 0, 0, 0);
                     }
                 }
             }
