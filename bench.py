@@ -51,7 +51,9 @@ HEADLINE = "fp6_4096x4096_bs8"
 # for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
     "fp6_4096x4096_bs8": 13241840,
-    "fp6_28672x8192_bs32": 182294683,  # measured with the stream kernel; the tile kernel now serves this shape
+    "fp6_8192x8192_bs8": 51572091,
+    "fp6_28672x8192_bs32": 187771045,   # GEMM kernel only; its split-K reduction kernel is a separate dispatch
+    "fp6_8192x8192_bs512": 126075242,
 }
 
 
