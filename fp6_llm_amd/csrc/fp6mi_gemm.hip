@@ -108,6 +108,23 @@ __device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
 // activations L2 -> VGPR directly in MFMA B-operand order (reused for the RT row tiles); the partial accumulators are
 // summed through LDS.  With PF the loads of the next K block are issued before the current one is consumed.
 // ---------------------------------------------------------------------------------------------------------------
+// Batches of at most 8 leave MFMA B columns 8..15 unused, and with them the lanes that would load those columns.  Those
+// lanes fetch the operand of the FOLLOWING MFMA step instead: lane (col, q) reads batch row col % 8 at step offset col / 8,
+// so one instruction brings two steps and touches whole 128-byte lines; a DPP rotation of each 16-lane row by 8 then moves
+// the second step's data down to columns 0..7.  Columns 8..15 end up holding the other step's (real, finite) data and only
+// feed output columns that are never stored.  (Four or eight steps per load for batches <= 4 or <= 2 measured no faster.)
+template <int NT> __device__ __forceinline__ void load_x_paired(v8h (&x)[8][NT], const half_t *src)
+{
+#pragma unroll
+    for (int sl = 0; sl < 4; sl++) {
+        v4u v = *reinterpret_cast<const v4u *>(src + 64 * sl), w;
+#pragma unroll
+        for (int i = 0; i < 4; i++) w[i] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[i], 0x128, 0xf, 0xf, false); // row_ror:8
+        x[2 * sl][0]     = __builtin_bit_cast(v8h, v);
+        x[2 * sl + 1][0] = __builtin_bit_cast(v8h, w);
+    }
+}
+
 template <int XB, int NT, int RT> struct Stage {
     WFrag<XB> w[RT];
     v8h       x[8][NT];
@@ -115,7 +132,7 @@ template <int XB, int NT, int RT> struct Stage {
 
 template <int XB, int NT, int RT>
 __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
-                                           const half_t *const (&xrow)[NT], int q, uint32_t K)
+                                           const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack, const half_t *xrow_packed)
 {
 #ifndef FP6MI_EXP_XFIRST
 #pragma unroll
@@ -125,6 +142,9 @@ __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t 
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
     // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
+    if (NT == 1 && xpack && (u + 1) * 256 <= K) { // uniform
+        load_x_paired(st.x, xrow_packed + u * 256);
+    } else
     if ((u + 1) * 256 <= K) { // uniform: whole block inside K, one base address and immediate offsets
 #pragma unroll
         for (int s = 0; s < 8; s++)
@@ -197,6 +217,10 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         uint32_t n = nbase + 16 * t + col;
         xrow[t]    = X + (size_t)(n < N ? n : N - 1) * K + 8 * q;
     }
+    // batches up to 8: two MFMA steps per activation load (see load_x_paired)
+    const bool    xpack = NT == 1 && N <= 8;
+    const int     prow = col & 7, pstep = col >> 3;
+    const half_t *xrow_packed = X + (size_t)((uint32_t)prow < N ? prow : N - 1) * K + 8 * q + 32 * pstep;
 
     // The epilogue gives thread e the output (row tile e/(256*NT), column tile, batch column, row e%16); its row scale is
     // fetched now so that no global load sits on the tail of the kernel.
@@ -214,12 +238,12 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     if (PF) {
         if (u < u1) {
             Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K);
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
             for (;;) {
                 uint32_t   un = u + WAVES;
                 const bool more = un < u1;
                 Stage<XB, NT, RT> nxt;
-                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, q, K);
+                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, q, K, xpack, xrow_packed);
                 consume_stage<XB, NT, RT>(cur, acc);
                 if (!more) break;
                 cur = nxt;
@@ -229,7 +253,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     } else {
         for (; u < u1; u += WAVES) {
             Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K);
+            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
             consume_stage<XB, NT, RT>(cur, acc);
         }
     }

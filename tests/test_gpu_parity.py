@@ -107,7 +107,7 @@ def test_config1_cpu_reference_case(E, M):
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
-@pytest.mark.parametrize("N", [1, 7, 8, 9, 16, 17, 33, 65, 129, 200])
+@pytest.mark.parametrize("N", [1, 2, 3, 4, 5, 7, 8, 9, 16, 17, 33, 65, 129, 200])
 def test_batch_edges(E, M, N):
     print("case batch edge", E, M, N, flush=True)
     OC, IC = 256, 512
