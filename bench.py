@@ -11,7 +11,8 @@ the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 
 
 Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth figure the reference's design is judged
 on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
-launch stream; `cpu_baseline` times the reference's CPU path (dequantize, then a torch CPU matmul) on this host.
+launch stream; `cpu_baseline` times the reference's CPU path (dequantize, then a torch CPU matmul) on this host;
+`detail.read_floor_us` is the time of a kernel that only reads the same weight buffers the same way (no arithmetic).
 --sweep additionally runs every benchmark configuration and writes gpurun_out/bench_sweep.jsonl.
 """
 import argparse
@@ -123,6 +124,46 @@ def time_steps(prob, steps, warmup, cold):
     return t1 - t0, e0.elapsed_time(e1)
 
 
+def read_floor_us(prob, steps, warmup):
+    """Time of a kernel that only reads the same weight buffers (same rotation, same graph protocol, same 128-bit
+    non-temporal loads and launch geometry as the small-batch GEMM): what any single-pass kernel over these bytes pays."""
+    import ctypes
+
+    import torch
+
+    path = os.path.join(ROOT, "fp6_llm_amd", "libfp6mi_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.fp6mi_probe_stream_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_void_p]
+    lib.fp6mi_probe_stream_read.restype = ctypes.c_int
+    sink = torch.zeros(16, dtype=torch.int32, device=prob.x.device)
+    nbytes = prob.weights[0].numel() * prob.weights[0].element_size()
+
+    def step(i):
+        w = prob.weights[i % prob.nbuf]
+        rc = lib.fp6mi_probe_stream_read(torch.cuda.current_stream().cuda_stream, w.data_ptr(), nbytes, sink.data_ptr())
+        assert rc == 0, rc
+
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for i in range(warmup):
+            step(i)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(steps):
+                step(warmup + i)
+        graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / steps
+
+
 def fp16_baseline_us(prob, steps, warmup):
     """FP16 GEMM of the same shape on the same GPU (torch F.linear = hipBLASLt/rocBLAS), weights rotating the same way:
     the counterpart of the reference's cuBLAS baseline (tests/python/kernel_test_fp6.py:45-62)."""
@@ -206,6 +247,11 @@ def run_workload(name, steps, warmup, device, with_fp16=True):
         "hbm_frac": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
         "splitK": prob.splitK, "weight_buffers": prob.nbuf, "weight_bytes": wb, "algorithmic_bytes": algorithmic_bytes(E, M, OC, IC, BS),
     }
+    floor = read_floor_us(prob, steps, warmup)
+    if floor is not None:
+        res["read_floor_us"] = round(floor, 3)               # a kernel that only reads these weight buffers once
+        res["read_floor_GBps"] = round(wb / floor / 1e3, 1)
+        res["frac_of_read_floor"] = round(floor / us, 4)
     if with_fp16:
         del prob.weights[2:]
         import torch
@@ -266,8 +312,9 @@ def main():
                 r, _ = run_workload(name, 100 if big else 300, 10, device)
                 f.write(json.dumps(r) + "\n")
                 f.flush()
-                print("%-22s %8.2f us  %7.0f GB/s (%.1f%% HBM)  %7.1f TFLOP/s  fp16 %8.2f us  x%.2f" % (
-                    name, r["us_per_gemm"], r["weight_GBps"], 100 * r["hbm_frac"], r["tflops"], r["fp16_gemm_us"], r["speedup_vs_fp16"]), file=sys.stderr, flush=True)
+                print("%-22s %8.2f us  %7.0f GB/s (%.1f%% HBM)  %7.1f TFLOP/s  read-only %7.2f us  fp16 %8.2f us  x%.2f" % (
+                    name, r["us_per_gemm"], r["weight_GBps"], 100 * r["hbm_frac"], r["tflops"], r.get("read_floor_us", float("nan")),
+                    r["fp16_gemm_us"], r["speedup_vs_fp16"]), file=sys.stderr, flush=True)
     print(json.dumps(line), flush=True)
 
 

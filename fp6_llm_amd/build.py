@@ -8,6 +8,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 SOURCES = [os.path.join(HERE, "csrc", "fp6mi_host.cpp"), os.path.join(HERE, "csrc", "fp6mi_gemm.hip")]
 OUTPUT = os.path.join(HERE, "libfp6mi.so")
+# measurement aid for the benchmark (a read-only streaming kernel); not linked into the engine
+PROBE_SOURCES = [os.path.join(HERE, "csrc", "stream_probe.hip")]
+PROBE_OUTPUT = os.path.join(HERE, "libfp6mi_probe.so")
 
 
 def hipcc_path():
@@ -17,19 +20,24 @@ def hipcc_path():
     raise RuntimeError("hipcc not found; the FPx engine cannot be built without the ROCm compiler")
 
 
-def build(verbose=False):
-    """Compiles every HIP/C++ source for gfx950 into libfp6mi.so (always recompiles)."""
+def _compile(sources, output, verbose):
     cmd = [hipcc_path(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
            # packed FP32 VALU forms are kept out of the generated code on this hardware pool
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-I" + os.path.join(ROOT, "include")] + SOURCES + ["-o", OUTPUT + ".tmp"]
+           "-I" + os.path.join(ROOT, "include")] + sources + ["-o", output + ".tmp"]
     res = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or res.returncode != 0:
         sys.stderr.write(res.stdout + res.stderr)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed building libfp6mi.so")
-    os.replace(OUTPUT + ".tmp", OUTPUT)
-    return OUTPUT
+        raise RuntimeError("hipcc failed building " + os.path.basename(output))
+    os.replace(output + ".tmp", output)
+    return output
+
+
+def build(verbose=False):
+    """Compiles every HIP/C++ source for gfx950 into libfp6mi.so and libfp6mi_probe.so (always recompiles)."""
+    _compile(PROBE_SOURCES, PROBE_OUTPUT, verbose)
+    return _compile(SOURCES, OUTPUT, verbose)
 
 
 if __name__ == "__main__":

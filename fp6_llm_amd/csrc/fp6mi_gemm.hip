@@ -106,7 +106,7 @@ __device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
 // A workgroup owns 16*RT output rows and 16*NT batch columns over the K blocks of its split; its wavefronts take the
 // blocks round-robin (K is split inside the workgroup), each streaming its weights HBM -> VGPR and its slice of the
 // activations L2 -> VGPR directly in MFMA B-operand order (reused for the RT row tiles); the partial accumulators are
-// summed through LDS.  With PF the loads of the next K block are issued before the current one is consumed.
+// summed through LDS.
 // ---------------------------------------------------------------------------------------------------------------
 // Batches of at most 8 leave MFMA B columns 8..15 unused, and with them the lanes that would load those columns.  Those
 // lanes fetch the operand of the FOLLOWING MFMA step instead: lane (col, q) reads batch row col % 8 at step offset col / 8,
@@ -134,11 +134,8 @@ template <int XB, int NT, int RT>
 __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
                                            const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack, const half_t *xrow_packed)
 {
-#ifndef FP6MI_EXP_XFIRST
 #pragma unroll
     for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
-#endif
-#ifndef FP6MI_EXP_NOX
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
     // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
@@ -160,16 +157,6 @@ __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t 
         }
     }
     __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
-#else
-#pragma unroll
-    for (int s = 0; s < 8; s++)
-#pragma unroll
-        for (int t = 0; t < NT; t++) { v8h o = { 1, 1, 1, 1, 1, 1, 1, 1 }; st.x[s][t] = o; }
-#endif
-#ifdef FP6MI_EXP_XFIRST
-#pragma unroll
-    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
-#endif
 }
 
 template <int XB, int NT, int RT>
@@ -186,7 +173,7 @@ __device__ __forceinline__ void consume_stage(const Stage<XB, NT, RT> &st, v4f (
     }
 }
 
-template <int XB, int NT, int RT, int WAVES, bool PF>
+template <int XB, int NT, int RT, int WAVES>
 __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
                                                             const half_t *__restrict__ X, half_t *__restrict__ C,
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
@@ -234,28 +221,12 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 
     // workgroups that share an L2 (ids congruent mod 8) start on different K blocks, so that the chip does not ask
     // the same activation lines of the same L2 channel at the same moment
-    uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES);
-    if (PF) {
-        if (u < u1) {
-            Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
-            for (;;) {
-                uint32_t   un = u + WAVES;
-                const bool more = un < u1;
-                Stage<XB, NT, RT> nxt;
-                if (more) load_stage<XB, NT, RT>(nxt, wgroup, tile_stride, un, lane, xrow, q, K, xpack, xrow_packed);
-                consume_stage<XB, NT, RT>(cur, acc);
-                if (!more) break;
-                cur = nxt;
-                u   = un;
-            }
-        }
-    } else {
-        for (; u < u1; u += WAVES) {
-            Stage<XB, NT, RT> cur;
-            load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
-            consume_stage<XB, NT, RT>(cur, acc);
-        }
+    // One K block at a time and no register double-buffering: the other wavefronts of the workgroup keep the memory system
+    // busy while this one converts, and a second stage in registers measured slower at every size.
+    for (uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES); u < u1; u += WAVES) {
+        Stage<XB, NT, RT> cur;
+        load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
+        consume_stage<XB, NT, RT>(cur, acc);
     }
 
     // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
@@ -370,11 +341,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 
     auto load_w = [&](WFrag<XB>(&dst)[RT], uint32_t c0) {
         const uint32_t u = c0 + wk;
-#ifdef FP6MI_EXP_NOWT
-        if (u == u0 + wk) {
-#else
         if (u < u1) {
-#endif
 #pragma unroll
             for (int r = 0; r < RT; r++) dst[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
         }
@@ -392,9 +359,6 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         xlds[j] = (p >> 5) * kXsRowBytes + (p & 31) * 16;
     }
     auto load_x = [&](uint32_t c0) {
-#ifdef FP6MI_EXP_NOXT
-        return;
-#endif
         if ((c0 + WK) * 256 <= K && c0 + WK <= u1) { // uniform: the whole chunk lies inside K and inside the split
 #pragma unroll
             for (int j = 0; j < kPerThread; j++)
@@ -412,9 +376,6 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         }
     };
     auto store_x = [&](int buf) {
-#ifdef FP6MI_EXP_NOXT
-        return;
-#endif
 #pragma unroll
         for (int j = 0; j < kPerThread; j++)
             if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) *reinterpret_cast<v4u *>(lds + buf * kBufBytes + xlds[j]) = xr[j];
@@ -446,11 +407,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
                     for (int s = 0; s < 4; s++) {
                         v8h b[NT];
 #pragma unroll
-#ifdef FP6MI_EXP_NOLDS
-                        for (int t = 0; t < NT; t++) { v8h o = { 1, 1, 1, 1, 1, 1, 1, 1 }; b[t] = o * (half_t)(float)(t + s + lane); }
-#else
                         for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xs + t * 16 * kXsRowBytes + (4 * h + s) * 64);
-#endif
 #pragma unroll
                         for (int r = 0; r < RT; r++)
 #pragma unroll
@@ -636,13 +593,13 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int XB, int NT, int RT, int WAVES, bool PF>
+template <int XB, int NT, int RT, int WAVES>
 int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
                   int splitK)
 {
     uint32_t units = (uint32_t)((K + 255) / 256);
     dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    hipLaunchKernelGGL((gemm_stream<XB, NT, RT, WAVES, PF>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
+    hipLaunchKernelGGL((gemm_stream<XB, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
                        static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M,
                        (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
     return (int)hipGetLastError();
@@ -673,9 +630,6 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
 }
 
 // kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
-#ifndef FP6MI_PF
-#define FP6MI_PF false
-#endif
 struct LaunchCfg { int kind, nt, rt, wr, wk; };
 
 inline size_t pow2_floor(size_t v)
@@ -750,7 +704,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
 {
     if (c.kind == 0) {
 #define FP6MI_CASE(NT, RT, WV) \
-    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV, FP6MI_PF>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
         FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
