@@ -27,7 +27,7 @@ __all__ = [
     "linear_forward_eXmY_cuda", "weight_prepacking_eXmY_cpu", "weight_dequant_eXmY_cpu",
     "Num_Wave", "HeuristicFuntion_SplitK",
     "weight_prepacking_native_cpu", "to_native", "linear_forward_native", "native_bytes",
-    "weight_dequant_native_cuda", "heuristic_splitk_mi355x", "clear_caches",
+    "weight_dequant_native_cuda", "weight_quantize_native_cuda", "heuristic_splitk_mi355x", "clear_caches",
 ]
 
 MI355X_CUS = 256
@@ -164,6 +164,29 @@ def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC
         _lib.check(_lib.lib().fp6mi_dequant_native_gpu(EXPONENT, MANTISSA, stream, out.data_ptr(), native_weight.data_ptr(),
                                                        fp16_scale.contiguous().data_ptr(), OC, IC), "fp6mi_dequant_native_gpu")
     return out
+
+
+_QUANT_DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
+
+
+def weight_quantize_native_cuda(EXPONENT, MANTISSA, weight):
+    """Float weights [OC, IC] (fp16, bf16 or fp32) on the GPU -> (native-layout int32 tensor, fp16 scales [OC]) on the same GPU:
+    per-row absmax scales, round to nearest with ties to the even code, clamped at the format maximum.  Gives the same
+    bits as quant.quantize_rowwise + quant.pack_raw + weight_prepacking_native_cpu on the host, without leaving the device."""
+    _bits(EXPONENT, MANTISSA)
+    if weight.device.type != "cuda" or weight.dim() != 2 or weight.dtype not in _QUANT_DTYPES:
+        raise ValueError("weight must be a 2-D fp16, bf16 or fp32 tensor on the GPU")
+    OC, IC = weight.shape
+    if OC % 16 or IC % 64:
+        raise ValueError("weight_quantize_native_cuda needs OC %% 16 == 0 and IC %% 64 == 0, got [%d, %d]" % (OC, IC))
+    weight = weight.contiguous()
+    native = torch.empty(native_bytes(EXPONENT, MANTISSA, OC, IC) // 4, dtype=torch.int32, device=weight.device)
+    scales = torch.empty(OC, dtype=torch.float16, device=weight.device)
+    with torch.cuda.device(weight.device):
+        stream = torch.cuda.current_stream().cuda_stream
+        _lib.check(_lib.lib().fp6mi_quantize_native_gpu(EXPONENT, MANTISSA, stream, native.data_ptr(), scales.data_ptr(), weight.data_ptr(),
+                                                        _QUANT_DTYPES[weight.dtype], OC, IC), "fp6mi_quantize_native_gpu")
+    return native, scales
 
 
 # ----------------------------------------------------------------------------------------------------------------

@@ -504,6 +504,48 @@ __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, 
     }
 }
 
+// Writes the 64 codes of one lane (c[8*s + j] = code of its row at column 32*s + 8*q + j of the K block) as the lane's
+// 12 (FP6) or 10 (FP5) dwords of a native block.
+template <int XB> __device__ __forceinline__ void store_native_lane(const uint8_t (&c)[64], uint8_t *dst, int lane)
+{
+    if (XB == 6) {
+        uint32_t d[12];
+        for (int h = 0; h < 2; h++) {
+            uint64_t accb = 0;
+            int      nb = 0, w = 0;
+            for (int i = 0; i < 32; i++) {
+                accb |= (uint64_t)c[32 * h + i] << nb;
+                nb += 6;
+                if (nb >= 32) { d[6 * h + w++] = (uint32_t)accb; accb >>= 32; nb -= 32; }
+            }
+        }
+        for (int i = 0; i < 3; i++) {
+            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
+            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        }
+    } else {
+        const int slot[4] = { 2, 1, 3, 0 };
+        uint32_t  d[10];
+        d[8] = d[9] = 0;
+        for (int s = 0; s < 8; s++) {
+            uint32_t word = 0;
+            for (int p = 0; p < 4; p++) {
+                uint32_t lo = c[8 * s + 2 * p], hi = c[8 * s + 2 * p + 1];
+                int      pp = 4 * (s & 3) + p;
+                word |= (lo & 15u) << (4 * slot[p]) | (hi & 15u) << (4 * (slot[p] + 4));
+                d[8 + (s >> 2)] |= ((lo >> 4) & 1u) << (15 - pp) | ((hi >> 4) & 1u) << (31 - pp);
+            }
+            d[s] = word;
+        }
+        for (int i = 0; i < 2; i++) {
+            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
+            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        }
+        v2u sv = { d[8], d[9] };
+        reinterpret_cast<v2u *>(dst + 2048)[lane] = sv;
+    }
+}
+
 // Reference layout -> native layout on the device.  One thread per (row tile, K block, lane): it gathers its 64
 // codes bit piece by bit piece from the reference's segment arrays and writes its 10 or 12 native dwords.
 __constant__ uint8_t kInvOrder4[8]  = { 4, 0, 6, 2, 5, 1, 7, 3 };
@@ -550,43 +592,96 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
             c[8 * s + j] = (uint8_t)code;
         }
     }
-    uint8_t *dst = native + (size_t)blk * Fmt<XB>::block_bytes;
-    if (XB == 6) {
-        uint32_t d[12];
-        for (int h = 0; h < 2; h++) {
-            uint64_t accb = 0;
-            int      nb = 0, w = 0;
-            for (int i = 0; i < 32; i++) {
-                accb |= (uint64_t)c[32 * h + i] << nb;
-                nb += 6;
-                if (nb >= 32) { d[6 * h + w++] = (uint32_t)accb; accb >>= 32; nb -= 32; }
-            }
-        }
-        for (int i = 0; i < 3; i++) {
-            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
-            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
-        }
-    } else {
-        const int slot[4] = { 2, 1, 3, 0 };
-        uint32_t  d[10];
-        d[8] = d[9] = 0;
-        for (int s = 0; s < 8; s++) {
-            uint32_t word = 0;
-            for (int p = 0; p < 4; p++) {
-                uint32_t lo = c[8 * s + 2 * p], hi = c[8 * s + 2 * p + 1];
-                int      pp = 4 * (s & 3) + p;
-                word |= (lo & 15u) << (4 * slot[p]) | (hi & 15u) << (4 * (slot[p] + 4));
-                d[8 + (s >> 2)] |= ((lo >> 4) & 1u) << (15 - pp) | ((hi >> 4) & 1u) << (31 - pp);
-            }
-            d[s] = word;
-        }
-        for (int i = 0; i < 2; i++) {
-            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
-            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
-        }
-        v2u sv = { d[8], d[9] };
-        reinterpret_cast<v2u *>(dst + 2048)[lane] = sv;
+    store_native_lane<XB>(c, native + (size_t)blk * Fmt<XB>::block_bytes, lane);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// Quantizer on the device: float weights [M,K] (fp16, bf16 or fp32) -> per-row fp16 scales + native-layout FPx codes.
+// Same arithmetic as the host quantizer of this package, so that both give identical bits:
+//   scale[row] = fp16_rn(absmax(row) / max_value) (1.0 where that rounds to zero), computed from a double quotient;
+//   code       = nearest representable magnitude to |w / scale| (a double quotient, clamped at max_value), ties to the even
+//                code, with the sign bit of w.
+// (The reference's only quantizer truncates and is not wired to any API: fp6_llm/csrc/utils/weight_quant.h:9-105.)
+// ---------------------------------------------------------------------------------------------------------------
+template <typename T> __device__ __forceinline__ float to_float(T v);
+template <> __device__ __forceinline__ float to_float<half_t>(half_t v) { return (float)v; }
+template <> __device__ __forceinline__ float to_float<float>(float v) { return v; }
+struct bf16_t { uint16_t bits; };
+template <> __device__ __forceinline__ float to_float<bf16_t>(bf16_t v) { return __builtin_bit_cast(float, (uint32_t)v.bits << 16); }
+
+// round-to-nearest-even of a non-negative double to fp16 without passing through float (no double rounding)
+__device__ __forceinline__ half_t half_rn_from_double(double q)
+{
+    if (!(q > 0.0)) return (half_t)0.0f;
+    int e = ilogb(q);                               // q = 1.xxx * 2^e
+    int ulp_exp = (e < -14 ? -14 : e) - 10;          // fp16 spacing at q (subnormals share the spacing 2^-24)
+    double r = rint(scalbn(q, -ulp_exp));            // exact scaling, then round to nearest even integer
+    double v = scalbn(r, ulp_exp);                   // representable in fp16 unless it overflows
+    return v >= 65520.0 ? (half_t)__builtin_inff() : (half_t)(float)v;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void quant_row_scales(half_t *__restrict__ scales, const T *__restrict__ Wf, uint32_t M, uint32_t K,
+                                                       double max_value)
+{
+    const int      lane = threadIdx.x & 63;
+    const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (row >= M) return;
+    const T *p = Wf + (size_t)row * K;
+    float    amax = 0.f;
+    for (uint32_t k = lane * 8; k < K; k += 512)
+#pragma unroll
+        for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(to_float<T>(p[k + j])));
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
+    if (lane == 0) {
+        half_t sc = half_rn_from_double((double)amax / max_value);
+        scales[row] = (float)sc == 0.f ? (half_t)1.0f : sc;
     }
+}
+
+// index (= magnitude bits of the code) of the representable magnitude nearest to a, 0 <= a <= max_value
+template <int XB> __device__ __forceinline__ uint32_t nearest_magnitude(double a)
+{
+    constexpr int bias = XB == 6 ? 3 : 1; // e3m2 / e2m2
+    int           e = a > 0.0 ? ilogb(a) : -1000;
+    if (e < 1 - bias) e = 1 - bias;                        // subnormals use the spacing of the first binade
+    double   t = scalbn(a, 2 - e);                         // in units of the spacing 2^(e-2): [0,4) subnormal, [4,8) normal
+    double   fl = floor(t), frac = t - fl;
+    uint32_t lo = (uint32_t)fl + (e > 1 - bias || fl >= 4.0 ? (uint32_t)(e + bias - 1) * 4u : 0u);
+    // (normal: index = (e+bias)*4 + (fl-4); subnormal: index = fl, and fl == 4 cannot happen there)
+    if (frac > 0.5 || (frac == 0.5 && (lo & 1u))) lo += 1;
+    return lo;
+}
+
+template <int XB, typename T>
+__global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ native, const half_t *__restrict__ scales,
+                                                      const T *__restrict__ Wf, uint32_t M, uint32_t K, uint32_t units, double max_value)
+{
+    const int      lane = threadIdx.x & 63;
+    const uint32_t blk = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (blk >= (M / 16) * units) return;
+    const uint32_t R = blk / units, U = blk % units;
+    const int      m = lane & 15, q = lane >> 4;
+    const uint32_t row = R * 16 + m;
+    const double   sc = (double)(float)scales[row];
+    const T       *p = Wf + (size_t)row * K;
+    uint8_t        c[64];
+#pragma unroll 1
+    for (int s = 0; s < 8; s++) {
+        const uint32_t k0 = U * 256 + 32 * s + 8 * q;
+        for (int j = 0; j < 8; j++) {
+            uint32_t code = 0;
+            if (k0 + j < K) {
+                float  w = to_float<T>(p[k0 + j]);
+                double a = fabs((double)w / sc);
+                if (!(a <= max_value)) a = max_value; // clamps, and sends NaN to the maximum like a saturating cast
+                code = nearest_magnitude<XB>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (XB - 1));
+            }
+            c[8 * s + j] = (uint8_t)code;
+        }
+    }
+    store_native_lane<XB>(c, native + (size_t)blk * Fmt<XB>::block_bytes, lane);
 }
 
 // ------------------------------------------------------------------------------------------------ launch helpers
@@ -940,6 +1035,41 @@ int fp6mi_dequant_native_gpu(int E, int Mb, void *stream, void *out, const void 
     else
         hipLaunchKernelGGL(dequant_native<5>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
                            static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
+    return (int)hipGetLastError();
+}
+
+int fp6mi_quantize_native_gpu(int E, int Mb, void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (!native || !scales || !weights) return FP6MI_ERR_NULL;
+    if (dtype < 0 || dtype > 2) return FP6MI_ERR_FORMAT;
+    if (M == 0 || M % 16 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu) return FP6MI_ERR_SHAPE;
+    if (!aligned16(native) || !aligned16(weights)) return FP6MI_ERR_ALIGN;
+    const uint32_t units = (uint32_t)((K + 255) / 256);
+    const size_t   blocks = (M / 16) * units;
+    const dim3     grid_rows((uint32_t)((M + 3) / 4)), grid_blocks((uint32_t)((blocks + 3) / 4));
+    const double   max_value = E == 3 ? 28.0 : 7.0;
+    hipStream_t    st = static_cast<hipStream_t>(stream);
+    uint8_t       *nat = static_cast<uint8_t *>(native);
+    half_t        *sc = static_cast<half_t *>(scales);
+#define FP6MI_QUANT(T)                                                                                                                    \
+    do {                                                                                                                                  \
+        hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, static_cast<const T *>(weights), (uint32_t)M, (uint32_t)K, \
+                           max_value);                                                                                                    \
+        if (E == 3)                                                                                                                       \
+            hipLaunchKernelGGL((quant_to_native<6, T>), grid_blocks, dim3(256), 0, st, nat, sc, static_cast<const T *>(weights),          \
+                               (uint32_t)M, (uint32_t)K, units, max_value);                                                               \
+        else                                                                                                                              \
+            hipLaunchKernelGGL((quant_to_native<5, T>), grid_blocks, dim3(256), 0, st, nat, sc, static_cast<const T *>(weights),          \
+                               (uint32_t)M, (uint32_t)K, units, max_value);                                                               \
+    } while (0)
+    if (dtype == 0)
+        FP6MI_QUANT(half_t);
+    else if (dtype == 1)
+        FP6MI_QUANT(bf16_t);
+    else
+        FP6MI_QUANT(float);
+#undef FP6MI_QUANT
     return (int)hipGetLastError();
 }
 

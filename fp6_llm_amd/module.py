@@ -8,7 +8,7 @@ import torch
 
 from . import quant
 from . import (MI355X_CUS, heuristic_splitk_mi355x, linear_forward_native, native_bytes, to_native,
-               weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu)
+               weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu, weight_quantize_native_cuda)
 
 _MAGIC = b"FP6MI\x00\x01\x00"   # name, NUL, layout version 1, reserved
 
@@ -50,10 +50,38 @@ class FPxLinear(torch.nn.Module):
 
     @classmethod
     def from_float(cls, weight, exponent=3, mantissa=2, bias=None, split_k=None):
-        """Quantizes a float [OC, IC] weight row-wise (round to nearest even, absmax scales) and packs it."""
+        """Quantizes a float [OC, IC] weight row-wise (round to nearest even, absmax scales) and packs it; a weight that
+        already lives on the GPU is quantized there (same bits as the host path)."""
+        if weight.device.type == "cuda" and weight.dtype in (torch.float16, torch.bfloat16, torch.float32):
+            native, scales = weight_quantize_native_cuda(exponent, mantissa, weight.detach())
+            m = cls(weight.shape[1], weight.shape[0], exponent, mantissa, bias, split_k).to(weight.device)
+            m.weight_native.copy_(native)
+            m.scales.copy_(scales)
+            return m
         codes, scales = quant.quantize_rowwise(weight.detach().float().cpu().numpy(), exponent, mantissa)
         raw = torch.from_numpy(quant.pack_raw(codes, exponent, mantissa))
         return cls.from_raw(raw, torch.from_numpy(scales), exponent, mantissa, bias, split_k)
+
+    @classmethod
+    def fused(cls, layers, split_k=None):
+        """One layer that computes several layers over the same input in a single launch (fused QKV, gate + up): its output
+        is the concatenation of theirs along the feature axis.  Rows are independent in the native layout (16-row tiles
+        are stored one after another), so fusing is a concatenation of the weight buffers, scales and biases."""
+        layers = list(layers)
+        first = layers[0]
+        for l in layers:
+            if (l.in_features, l.exponent, l.mantissa) != (first.in_features, first.exponent, first.mantissa):
+                raise ValueError("fused layers must share in_features and the weight format")
+            if (l.bias is None) != (first.bias is None):
+                raise ValueError("fused layers must all have a bias or all have none")
+            if l.weight_native.device != first.weight_native.device:
+                raise ValueError("fused layers must live on one device")
+        bias = None if first.bias is None else torch.cat([l.bias for l in layers])
+        m = cls(first.in_features, sum(l.out_features for l in layers), first.exponent, first.mantissa, bias, split_k)
+        m = m.to(first.weight_native.device)
+        m.weight_native.copy_(torch.cat([l.weight_native for l in layers]))
+        m.scales.copy_(torch.cat([l.scales for l in layers]))
+        return m
 
     def forward(self, x):
         lead = x.shape[:-1]

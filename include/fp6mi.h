@@ -108,6 +108,15 @@ int fp6mi_relayout_ref_to_native_gpu(int E, int Mbits, void *stream, void *nativ
 int fp6mi_dequant_native_gpu(int E, int Mbits, void *stream, void *out_f16_dev, const void *W_native_dev,
                              const void *scales_f16_dev, size_t M, size_t K);
 
+/* Device-side quantizer: float weights [M,K] (dtype 0 = fp16, 1 = bf16, 2 = fp32; device pointer, row-major) to
+ * per-row fp16 scales [M] (absmax / format maximum, 1.0 for an all-zero row) and native-layout FPx codes
+ * (round to nearest, ties to the even code, clamped at the format maximum).  The step BEFORE the reference's path: the
+ * reference only ships a truncating fp16->fp6 cast that no API calls (fp6_llm/csrc/utils/weight_quant.h:9-105,
+ * "weight_prepacking_fp16_to_fp6"); this replaces quantize-on-CPU + weight_matrix_prepacking for checkpoints that are
+ * already on the GPU.  M % 16 == 0 (256 for the GEMM), K % 64 == 0; native_dev holds fp6mi_native_bytes(E,M,...) bytes. */
+int fp6mi_quantize_native_gpu(int E, int Mbits, void *stream, void *native_dev, void *scales_f16_dev,
+                              const void *weights_dev, int dtype, size_t M, size_t K);
+
 #ifdef __cplusplus
 }
 #endif

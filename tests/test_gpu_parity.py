@@ -294,6 +294,59 @@ def test_module_forward():
         check_close(y.reshape(10, 512).cpu().numpy(), ref, "module e%dm%d" % (E, M))
 
 
+# ------------------------------------------------------------------------------------------------ device-side quantizer
+def _awkward_weights(seed, OC, IC, dtype):
+    """Gaussian weights with the cases a quantizer gets wrong: an all-zero row, a row of tiny values whose scale rounds to
+    an fp16 subnormal, a huge row, negative zeros, and values placed exactly on rounding ties of the scaled grid."""
+    w = synth.normal(seed, (OC, IC)).astype(np.float32)
+    w[1, :] = 0.0
+    w[2, :] *= 1e-7
+    w[3, :] *= 3000.0
+    w[4, ::3] = -0.0
+    w[5, :] = 0.0
+    w[5, 0] = 28.0                                            # scale exactly 1.0: the row below sits on ties and exact values
+    w[5, 1:65] = np.arange(64, dtype=np.float32) * 0.4375     # multiples of 7/16: many land midway between codes
+    w[6, :] = -w[5, :]
+    t = torch.from_numpy(w).to(dtype)
+    return t
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("OC,IC", [(256, 512), (512, 320), (1024, 4096)])
+def test_device_quantizer_matches_host_bits(E, M, dtype, OC, IC):
+    print("case device quantizer", E, M, dtype, OC, IC, flush=True)
+    w = _awkward_weights(41, OC, IC, dtype)
+    native, scales = fp6.weight_quantize_native_cuda(E, M, w.to(DEV))
+    codes, sc_host = quant.quantize_rowwise(w.float().numpy().astype(np.float64), E, M)
+    native_host = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M)))
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), sc_host.view(np.uint16))
+    assert torch.equal(native.cpu(), native_host)
+
+
+def test_device_quantizer_rejects_bad_arguments():
+    with pytest.raises(ValueError):
+        fp6.weight_quantize_native_cuda(3, 2, torch.zeros(256, 100, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError):
+        fp6.weight_quantize_native_cuda(3, 2, torch.zeros(256, 128, dtype=torch.float64, device=DEV))
+    with pytest.raises(ValueError):
+        fp6.weight_quantize_native_cuda(4, 3, torch.zeros(256, 128, dtype=torch.float16, device=DEV))
+    with pytest.raises(ValueError):
+        fp6.weight_quantize_native_cuda(3, 2, torch.zeros(256, 128, dtype=torch.float16))
+
+
+def test_module_from_float_on_device_equals_host_path():
+    from fp6_llm_amd import module
+    w = torch.from_numpy(synth.normal(51, (512, 1024))).half()
+    for (E, M) in FORMATS:
+        host = module.FPxLinear.from_float(w, E, M)
+        dev = module.FPxLinear.from_float(w.to(DEV), E, M)
+        assert torch.equal(dev.weight_native.cpu(), host.weight_native)
+        assert torch.equal(dev.scales.cpu(), host.scales)
+        x = torch.from_numpy(synth.activations(52, 8, 1024)).to(DEV)
+        assert torch.equal(dev(x), host.to(DEV)(x))
+
+
 # ------------------------------------------------------------------------------------------------ benchmark configs
 def _bench_case(E, M, OC, IC, BS, seed, gaussian, act_sigma=1.0, splitKs=(None,)):
     print("case bench config", E, M, OC, IC, BS, flush=True)

@@ -244,3 +244,19 @@ def test_module_construction_routes_agree():
     assert torch.equal(c.weight_native, fp6.weight_prepacking_native_cpu(3, 2, torch.from_numpy(quant.pack_raw(codes, 3, 2))))
     with pytest.raises(ValueError):
         module.FPxLinear(100, 256)
+
+
+def test_fused_layers_are_the_concatenation():
+    """Fusing layers over one input = quantizing the row-concatenated weight: native tiles are stored row tile after row tile."""
+    from fp6_llm_amd import module
+    for (E, M) in ((3, 2), (2, 2)):
+        ws = [torch.from_numpy(synth.normal(61 + i, (oc, 320))).float() for i, oc in enumerate((256, 512, 256))]
+        bs = [torch.from_numpy(synth.normal(71 + i, (w.shape[0],))).half() for i, w in enumerate(ws)]
+        parts = [module.FPxLinear.from_float(w, E, M, bias=b) for w, b in zip(ws, bs)]
+        fused = module.FPxLinear.fused(parts)
+        whole = module.FPxLinear.from_float(torch.cat(ws), E, M, bias=torch.cat(bs))
+        assert fused.out_features == 1024 and fused.in_features == 320
+        assert torch.equal(fused.weight_native, whole.weight_native)
+        assert torch.equal(fused.scales, whole.scales) and torch.equal(fused.bias, whole.bias)
+    with pytest.raises(ValueError):
+        module.FPxLinear.fused([module.FPxLinear.from_float(ws[0], 3, 2), module.FPxLinear.from_float(ws[0], 2, 2)])
