@@ -6,9 +6,10 @@
 //   launchers     <- fpx_linear_kernel        fp6_llm/csrc/fp6_linear.cu:44-102
 // The design is not a translation: weights use the native layout described in fp6mi_host.cpp, go from HBM straight
 // to VGPRs with 128-bit non-temporal loads, FP6 codes are converted by the CDNA4 instruction
-// v_cvt_scalef32_pk32_f16_bf6 (BF6 = e3m2, bias 3, no inf/nan: the very format of the reference), FP5 codes by
-// shift/mask into fp16 bit patterns, and v_mfma_f32_16x16x32_f16 accumulates in FP32.  The per-row scale (and the
-// 2^14 exponent rebias of FP5) is applied once to the FP32 sums instead of to every weight.
+// v_cvt_scalef32_pk32_f16_bf6 (BF6 = e3m2, bias 3, no inf/nan: the very format of the reference), FP5 codes by the same
+// instruction after a zero bit is slipped in above their exponent (an e2m2 code read as e3m2 is a quarter of its value),
+// and v_mfma_f32_16x16x32_f16 accumulates in FP32.  The per-row scale (and the factor 4 of FP5) is applied once to the
+// FP32 sums instead of to every weight.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
@@ -30,7 +31,7 @@ constexpr int kWave = 64;
 
 template <int XB> struct Fmt;
 template <> struct Fmt<6> { static constexpr int block_bytes = 3072; static constexpr float post_scale = 1.0f; };
-template <> struct Fmt<5> { static constexpr int block_bytes = 2560; static constexpr float post_scale = 16384.0f; };
+template <> struct Fmt<5> { static constexpr int block_bytes = 2560; static constexpr float post_scale = 4.0f; };
 
 // The weights of one lane for one 16x256 block, as loaded from memory.
 template <int XB> struct WFrag;
@@ -58,7 +59,7 @@ template <> __device__ __forceinline__ WFrag<5> load_wfrag<5>(const uint8_t *blo
 }
 
 // A operands (8 halfs = k 8q..8q+7 of this lane's row) of the eight MFMA steps of a block.
-// FP6: exact values.  FP5: values times 2^-14 (fp16 subnormals included; the MFMA does not flush them).
+// FP6: exact values.  FP5: a quarter of the values (exact; the epilogue multiplies the sums by 4).
 template <int XB> struct AOps { v8h s[8]; };
 
 __device__ __forceinline__ v8h slice8(const v32h &v, int i)
@@ -84,19 +85,23 @@ __device__ __forceinline__ void convert(const WFrag<6> &f, AOps<6> &o)
     }
 }
 
+// FP5: 32 codes are stored in five dwords; the sixth dword of the 6-bit string the conversion instruction reads is parked
+// in the fixed-zero bits ("holes", bit 4 of every 6-bit field) of the other five and is put back here (layout: fp6mi_host.cpp).
+__device__ __forceinline__ v6u fp5_expand(uint32_t s0, uint32_t s1, uint32_t s2, uint32_t s3, uint32_t s4)
+{
+    constexpr uint32_t A = 0x10410410u, B = 0x04104104u, C = 0x41041041u;
+    uint32_t lo = (s0 & A) | (s1 & B), hi = (s2 & C) | (s3 & A) | (s4 & B);
+    return (v6u){ s0 & ~A, s1 & ~B, s2 & ~C, s3 & ~A, s4 & ~B, (hi << 1) | lo };
+}
+
 __device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
 {
-    constexpr uint32_t kNib = 0x0F000F00u, kSign = 0x80008000u;
+    v32h h0 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(fp5_expand(f.a[0], f.a[1], f.a[2], f.a[3], f.s[0]), 1.0f);
+    v32h h1 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(fp5_expand(f.b[0], f.b[1], f.b[2], f.b[3], f.s[1]), 1.0f);
 #pragma unroll
-    for (int s = 0; s < 8; s++) {
-        uint32_t w  = (s < 4) ? f.a[s & 3] : f.b[s & 3];
-        uint32_t sg = f.s[s >> 2] << (4 * (s & 3));
-        v4u      r;
-        r[0]   = (w & kNib) | (sg & kSign);
-        r[1]   = ((w << 4) & kNib) | ((sg << 1) & kSign);
-        r[2]   = ((w >> 4) & kNib) | ((sg << 2) & kSign);
-        r[3]   = ((w << 8) & kNib) | ((sg << 3) & kSign);
-        o.s[s] = __builtin_bit_cast(v8h, r);
+    for (int i = 0; i < 4; i++) {
+        o.s[i]     = slice8(h0, i);
+        o.s[4 + i] = slice8(h1, i);
     }
 }
 
@@ -267,18 +272,10 @@ __device__ __forceinline__ void convert_half(const WFrag<6> &f, int h, v8h (&o)[
 }
 __device__ __forceinline__ void convert_half(const WFrag<5> &f, int h, v8h (&o)[4])
 {
-    constexpr uint32_t kNib = 0x0F000F00u, kSign = 0x80008000u;
-    const v4u          nib = h == 0 ? f.a : f.b;
+    v6u  src = h == 0 ? fp5_expand(f.a[0], f.a[1], f.a[2], f.a[3], f.s[0]) : fp5_expand(f.b[0], f.b[1], f.b[2], f.b[3], f.s[1]);
+    v32h v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        uint32_t w = nib[i], sg = f.s[h] << (4 * i);
-        v4u      r;
-        r[0] = (w & kNib) | (sg & kSign);
-        r[1] = ((w << 4) & kNib) | ((sg << 1) & kSign);
-        r[2] = ((w >> 4) & kNib) | ((sg << 2) & kSign);
-        r[3] = ((w << 8) & kNib) | ((sg << 3) & kSign);
-        o[i] = __builtin_bit_cast(v8h, r);
-    }
+    for (int i = 0; i < 4; i++) o[i] = slice8(v, i);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -289,10 +286,11 @@ __device__ __forceinline__ void convert_half(const WFrag<5> &f, int h, v8h (&o)[
 // [WK][NT*16][256] in LDS (double-buffered, filled by fully coalesced 16-byte loads); wavefront (wr, wk) streams the
 // weights of its RT row tiles for K block wk straight from HBM into VGPRs (prefetched one chunk ahead), converts them
 // half a block at a time and runs RT*NT MFMAs per step against B operands read once per step from LDS.  The LDS row
-// stride is 256+8 halfs so that the eight lanes that read 16 bytes each in one LDS cycle fall in distinct banks.
+// stride is 256+16 halfs (544 bytes): measured on the MI355X, the 16-column x 4-k-group operand read (ds_read_b128) then runs at
+// the conflict-free rate of 7 cycles per wavefront, against 8.8 cycles at 528 bytes and 32 cycles without padding.
 // The WK partial accumulators are summed through LDS at the end (WK > 1), then scaled and stored.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kXsRowBytes = 528;
+constexpr int kXsRowBytes = 544;
 
 template <int XB, int NT, int RT, int WR, int WK>
 __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
@@ -524,24 +522,29 @@ template <int XB> __device__ __forceinline__ void store_native_lane(const uint8_
             reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
         }
     } else {
-        const int slot[4] = { 2, 1, 3, 0 };
-        uint32_t  d[10];
-        d[8] = d[9] = 0;
-        for (int s = 0; s < 8; s++) {
-            uint32_t word = 0;
-            for (int p = 0; p < 4; p++) {
-                uint32_t lo = c[8 * s + 2 * p], hi = c[8 * s + 2 * p + 1];
-                int      pp = 4 * (s & 3) + p;
-                word |= (lo & 15u) << (4 * slot[p]) | (hi & 15u) << (4 * (slot[p] + 4));
-                d[8 + (s >> 2)] |= ((lo >> 4) & 1u) << (15 - pp) | ((hi >> 4) & 1u) << (31 - pp);
+        constexpr uint32_t A = 0x10410410u, B = 0x04104104u, C = 0x41041041u;
+        uint32_t           S[2][5];
+        for (int h = 0; h < 2; h++) {
+            uint32_t D[6];
+            uint64_t accb = 0;
+            int      nb = 0, w = 0;
+            for (int i = 0; i < 32; i++) {
+                uint32_t code = c[32 * h + i], field = (code & 15u) | (((code >> 4) & 1u) << 5);
+                accb |= (uint64_t)field << nb;
+                nb += 6;
+                if (nb >= 32) { D[w++] = (uint32_t)accb; accb >>= 32; nb -= 32; }
             }
-            d[s] = word;
+            S[h][0] = D[0] | (D[5] & A);
+            S[h][1] = D[1] | (D[5] & B);
+            S[h][2] = D[2] | ((D[5] >> 1) & C);
+            S[h][3] = D[3] | ((D[5] >> 1) & A);
+            S[h][4] = D[4] | ((D[5] >> 1) & B);
         }
-        for (int i = 0; i < 2; i++) {
-            v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
-            reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        for (int h = 0; h < 2; h++) {
+            v4u v = { S[h][0], S[h][1], S[h][2], S[h][3] };
+            reinterpret_cast<v4u *>(dst)[h * 64 + lane] = v;
         }
-        v2u sv = { d[8], d[9] };
+        v2u sv = { S[0][4], S[1][4] };
         reinterpret_cast<v2u *>(dst + 2048)[lane] = sv;
     }
 }

@@ -245,15 +245,41 @@ int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, c
 // the twelve dwords d = 0..11 of a lane sit at byte (d/4)*1024 + 16*l + 4*(d%4), so three 16-byte loads per lane,
 // each contiguous over the wavefront, fetch a block.
 //
-// FP5_e2m2 block (2560 B), bit-sliced 4+1: dword s (0..7) of a lane holds the low four bits of the codes of step s,
-// code pair p = j/2 in nibble slots {2,6},{1,5},{3,7},{0,4} (low code in the lower slot; slot t = bits [4t,4t+4)),
-// so that `(word << {0,4,-4,8}) & 0x0F000F00` drops both nibbles of a pair onto bits 8..11 of the two fp16 halves;
-// dwords 8,9 hold the sign bits: pair pp = 4*(s%4) + p of half h = s/4 has its low/high sign at bits 15-pp / 31-pp of
-// dword 8+h, so `(word << pp) & 0x80008000` puts them on the fp16 sign bits.  Dwords 0..7 sit at
-// (d/4)*1024 + 16*l + 4*(d%4), dwords 8,9 at 2048 + 8*l + 4*(d-8).
+// FP5_e2m2 block (2560 B): the same two strings of 32 six-bit fields per lane, each field = the FP5 code with a zero
+// inserted above its two exponent bits (sign, 0, e1 e0 m1 m0): read as e3m2 that field is exactly a quarter of the e2m2
+// value, subnormals included, so the same hardware conversion applies.  A string would take six dwords D0..D5 with one
+// fixed-zero bit (a "hole", bit 4 of each field) per code; storage keeps five dwords S0..S4 per string by parking the 26
+// payload bits of D5 in the 26 holes of D0..D4, a residue class of bit positions per dword so that one mask (and one shared
+// shift) moves them back:
+//   S0 = D0 | (D5 & A)   S1 = D1 | (D5 & B)   S2 = D2 | ((D5 >> 1) & C)   S3 = D3 | ((D5 >> 1) & A)   S4 = D4 | ((D5 >> 1) & B)
+//   A = 0x10410410 (bits 4,10,..,28)   B = 0x04104104 (bits 2,8,..,26)   C = 0x41041041 (bits 0,6,..,30)
+//   D5 = (S0 & A) | (S1 & B) | (((S2 & C) | (S3 & A) | (S4 & B)) << 1),   Dk = Sk & ~(its hole mask)
+// Eleven integer instructions rebuild the six dwords of 32 codes.  Lane dwords: string h has S0..S3 in dwords 4h..4h+3
+// and S4 in dword 8+h; dwords 0..7 sit at (d/4)*1024 + 16*l + 4*(d%4), dwords 8,9 at 2048 + 8*l + 4*(d-8).
 size_t native_block_bytes(int x) { return x == 6 ? 3072 : 2560; }
 
-static const int kNibSlotLo[4] = { 2, 1, 3, 0 };
+static const uint32_t kHoleA = 0x10410410u, kHoleB = 0x04104104u, kHoleC = 0x41041041u;
+
+// 32 six-bit fields -> six dwords (little-endian bit string), and back
+static void fields_to_dwords(const uint8_t f[32], uint32_t o[6])
+{
+    for (int w = 0; w < 6; w++) o[w] = 0;
+    for (int i = 0; i < 32; i++) {
+        int      bit = 6 * i, w = bit >> 5, off = bit & 31;
+        uint32_t v   = f[i] & 63u;
+        o[w] |= v << off;
+        if (off > 26) o[w + 1] |= v >> (32 - off);
+    }
+}
+static void dwords_to_fields(const uint32_t o[6], uint8_t f[32])
+{
+    for (int i = 0; i < 32; i++) {
+        int      bit = 6 * i, w = bit >> 5, off = bit & 31;
+        uint32_t v   = o[w] >> off;
+        if (off > 26) v |= o[w + 1] << (32 - off);
+        f[i] = (uint8_t)(v & 63u);
+    }
+}
 
 static inline size_t native_dword_offset(int x, int lane, int d)
 {
@@ -263,56 +289,36 @@ static inline size_t native_dword_offset(int x, int lane, int d)
 
 static void native_pack_lane(int x, const uint8_t c[64], uint32_t d[12])
 {
-    if (x == 6) {
-        for (int h = 0; h < 2; h++) {
-            uint32_t *o = d + 6 * h;
-            for (int w = 0; w < 6; w++) o[w] = 0;
-            for (int i = 0; i < 32; i++) {
-                int      bit = 6 * i, w = bit >> 5, off = bit & 31;
-                uint32_t v   = c[32 * h + i] & 63u;
-                o[w] |= v << off;
-                if (off > 26) o[w + 1] |= v >> (32 - off);
-            }
-        }
-    } else {
-        d[8] = d[9] = 0;
-        for (int s = 0; s < 8; s++) {
-            uint32_t word = 0;
-            for (int p = 0; p < 4; p++) {
-                uint32_t lo = c[8 * s + 2 * p], hi = c[8 * s + 2 * p + 1];
-                word |= (lo & 15u) << (4 * kNibSlotLo[p]);
-                word |= (hi & 15u) << (4 * (kNibSlotLo[p] + 4));
-                int pp = 4 * (s % 4) + p;
-                d[8 + s / 4] |= ((lo >> 4) & 1u) << (15 - pp);
-                d[8 + s / 4] |= ((hi >> 4) & 1u) << (31 - pp);
-            }
-            d[s] = word;
+    for (int h = 0; h < 2; h++) {
+        if (x == 6) {
+            fields_to_dwords(c + 32 * h, d + 6 * h);
+        } else {
+            uint8_t  f[32];
+            uint32_t D[6];
+            for (int i = 0; i < 32; i++) f[i] = (uint8_t)((c[32 * h + i] & 15u) | (((c[32 * h + i] >> 4) & 1u) << 5));
+            fields_to_dwords(f, D);
+            d[4 * h + 0] = D[0] | (D[5] & kHoleA);
+            d[4 * h + 1] = D[1] | (D[5] & kHoleB);
+            d[4 * h + 2] = D[2] | ((D[5] >> 1) & kHoleC);
+            d[4 * h + 3] = D[3] | ((D[5] >> 1) & kHoleA);
+            d[8 + h]     = D[4] | ((D[5] >> 1) & kHoleB);
         }
     }
 }
 
 static void native_unpack_lane(int x, const uint32_t d[12], uint8_t c[64])
 {
-    if (x == 6) {
-        for (int h = 0; h < 2; h++) {
-            const uint32_t *o = d + 6 * h;
-            for (int i = 0; i < 32; i++) {
-                int      bit = 6 * i, w = bit >> 5, off = bit & 31;
-                uint32_t v   = o[w] >> off;
-                if (off > 26) v |= o[w + 1] << (32 - off);
-                c[32 * h + i] = (uint8_t)(v & 63u);
-            }
+    for (int h = 0; h < 2; h++) {
+        if (x == 6) {
+            dwords_to_fields(d + 6 * h, c + 32 * h);
+        } else {
+            const uint32_t S0 = d[4 * h], S1 = d[4 * h + 1], S2 = d[4 * h + 2], S3 = d[4 * h + 3], S4 = d[8 + h];
+            uint32_t       D[6] = { S0 & ~kHoleA, S1 & ~kHoleB, S2 & ~kHoleC, S3 & ~kHoleA, S4 & ~kHoleB,
+                                    (S0 & kHoleA) | (S1 & kHoleB) | (((S2 & kHoleC) | (S3 & kHoleA) | (S4 & kHoleB)) << 1) };
+            uint8_t        f[32];
+            dwords_to_fields(D, f);
+            for (int i = 0; i < 32; i++) c[32 * h + i] = (uint8_t)((f[i] & 15u) | (((f[i] >> 5) & 1u) << 4));
         }
-    } else {
-        for (int s = 0; s < 8; s++)
-            for (int p = 0; p < 4; p++) {
-                int      pp = 4 * (s % 4) + p;
-                uint32_t lo = (d[s] >> (4 * kNibSlotLo[p])) & 15u, hi = (d[s] >> (4 * (kNibSlotLo[p] + 4))) & 15u;
-                lo |= ((d[8 + s / 4] >> (15 - pp)) & 1u) << 4;
-                hi |= ((d[8 + s / 4] >> (31 - pp)) & 1u) << 4;
-                c[8 * s + 2 * p]     = (uint8_t)lo;
-                c[8 * s + 2 * p + 1] = (uint8_t)hi;
-            }
     }
 }
 

@@ -106,13 +106,17 @@ def test_native_fp6_lane_image_is_the_hardware_operand(E, M):
                 assert got == [int(v) for v in want[32 * h:32 * h + 32]]
         else:
             d = [blk[(i // 4) * 256 + lane * 4 + i % 4] for i in range(8)] + [blk[512 + lane * 2 + i] for i in range(2)]
-            slot = [2, 1, 3, 0]
-            for s in range(8):
-                for p in range(4):
-                    pp = 4 * (s % 4) + p
-                    lo = ((int(d[s]) >> (4 * slot[p])) & 15) | (((int(d[8 + s // 4]) >> (15 - pp)) & 1) << 4)
-                    hi = ((int(d[s]) >> (4 * (slot[p] + 4))) & 15) | (((int(d[8 + s // 4]) >> (31 - pp)) & 1) << 4)
-                    assert (lo, hi) == (int(want[8 * s + 2 * p]), int(want[8 * s + 2 * p + 1]))
+            # five stored dwords per string; the sixth dword of the 6-bit string sits in the fixed-zero bit of every field
+            A, B, C = 0x10410410, 0x04104104, 0x41041041
+            for h in range(2):
+                S = [int(d[4 * h + k]) for k in range(4)] + [int(d[8 + h])]
+                D = [S[0] & ~A, S[1] & ~B, S[2] & ~C, S[3] & ~A, S[4] & ~B,
+                     (S[0] & A) | (S[1] & B) | ((((S[2] & C) | (S[3] & A) | (S[4] & B)) << 1) & 0xFFFFFFFF)]
+                big = sum(D[w] << (32 * w) for w in range(6))
+                fields = [(big >> (6 * i)) & 63 for i in range(32)]
+                assert all((f >> 4) & 1 == 0 for f in fields)          # the inserted exponent bit
+                got = [(f & 15) | ((f >> 5) << 4) for f in fields]
+                assert got == [int(v) for v in want[32 * h:32 * h + 32]]
 
 
 def test_prepack_in_place_and_padding_is_zero():
@@ -260,3 +264,12 @@ def test_fused_layers_are_the_concatenation():
         assert torch.equal(fused.scales, whole.scales) and torch.equal(fused.bias, whole.bias)
     with pytest.raises(ValueError):
         module.FPxLinear.fused([module.FPxLinear.from_float(ws[0], 3, 2), module.FPxLinear.from_float(ws[0], 2, 2)])
+
+
+def test_e2m2_code_read_as_e3m2_is_a_quarter_of_its_value():
+    """What the FP5 native layout relies on: inserting a zero above the two exponent bits of an e2m2 code gives the e3m2
+    code of exactly a quarter of its value, for all 32 codes (subnormals and signed zeros included)."""
+    v5, v6 = oracle.value_table(2, 2), oracle.value_table(3, 2)
+    for code in range(32):
+        field = (code & 15) | ((code >> 4) << 5)
+        assert v6[field] * 4.0 == v5[code] and np.signbit(v6[field]) == np.signbit(v5[code])
