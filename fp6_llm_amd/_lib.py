@@ -43,6 +43,7 @@ def lib():
         "fp6mi_relayout_ref_to_native_gpu": (ci, [ci, ci, vp, vp, vp, sz, sz]),
         "fp6mi_dequant_native_gpu": (ci, [ci, ci, vp, vp, vp, vp, sz, sz]),
         "fp6mi_quantize_native_gpu": (ci, [ci, ci, vp, vp, vp, vp, ci, sz, sz]),
+        "fp6mi_query_launch": (ci, [ci, ci, sz, sz, sz, ci, ctypes.POINTER(ci)]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(L, name)
@@ -55,7 +56,7 @@ def lib():
 EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_prepack_ref", "fp6mi_dequant", "fp6mi_unpack_ref",
             "fp6mi_native_bytes", "fp6mi_prepack_native", "fp6mi_relayout_ref_to_native", "fp6mi_unpack_native",
             "fp6mi_heuristic_splitk", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_twin_evict", "fp6mi_twin_clear",
-            "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu"]
+            "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch"]
 
 
 def check(code, where):

@@ -749,6 +749,47 @@ inline size_t tile_k_parallelism(size_t M, size_t N, int cus)
 }
 constexpr size_t kMaxAutoSplitK = 8;
 
+// ---- measured launch shapes (generated by `python -m fp6_llm_amd.tune`, MI355X, 256 CUs) ----
+struct TuneCfg { uint8_t kind, nt, rt, wr, wk; uint16_t t; };              // t in 0.02 us; kind 255 = not measured
+struct TuneEntry { uint8_t xb; uint16_t m256, k64, n; TuneCfg sk[4]; };    // sk[i]: best shape for splitK = 1 << i
+const TuneEntry kTune[] = {
+    { 0, 0, 0, 0, { { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 } } }, // keeps the array non-empty
+#include "fp6mi_tuning.inc"
+};
+
+inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (16u * c.rt * (c.kind == 1 ? c.wr : 1u)) == 0; }
+
+// Nearest measured problem: the batch is rounded UP to a measured batch of the same kernel family (a shape's cost steps at
+// column-tile boundaries), M and K go to the nearest measured value in ratio, at most a factor 1.5 away.
+const TuneEntry *tune_lookup(int xbits, size_t M, size_t N, size_t K)
+{
+    struct Memo { int xb; size_t M, N, K; const TuneEntry *e; };
+    static thread_local Memo memo[8];
+    static thread_local unsigned next = 0;
+    for (const Memo &m : memo)
+        if (m.xb == xbits && m.M == M && m.N == N && m.K == K) return m.e;
+    const size_t count = sizeof(kTune) / sizeof(kTune[0]);
+    size_t       n_target = 0, n_max = 0;
+    for (size_t i = 1; i < count; i++) {
+        const TuneEntry &e = kTune[i];
+        if (e.xb != xbits || (e.n <= 16) != (N <= 16)) continue;
+        if (e.n >= N && (n_target == 0 || e.n < n_target)) n_target = e.n;
+        if (e.n > n_max) n_max = e.n;
+    }
+    if (n_target == 0) n_target = n_max; // batches beyond the largest measured one behave like it, only more column blocks
+    const TuneEntry *best = nullptr;
+    float            best_d = 0.f;
+    for (size_t i = 1; n_target && i < count; i++) {
+        const TuneEntry &e = kTune[i];
+        if (e.xb != xbits || e.n != n_target) continue;
+        float dm = std::fabs(std::log2((float)M / (256.f * e.m256))), dk = std::fabs(std::log2((float)K / (64.f * e.k64)));
+        if (dm > 0.585f || dk > 0.585f) continue;
+        if (!best || dm + dk < best_d) { best = &e; best_d = dm + dk; }
+    }
+    memo[next++ % 8] = Memo{ xbits, M, N, K, best };
+    return best;
+}
+
 // Launch shape for a given splitK.
 //  N <= 16: stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M; wavefronts
 //           per workgroup follow the K blocks of one split and the register budget (16 wavefronts leave 128 VGPRs each).
@@ -757,24 +798,45 @@ constexpr size_t kMaxAutoSplitK = 8;
 inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, int cus)
 {
     LaunchCfg c;
+    if (cus == 256 && (splitK == 1 || splitK == 2 || splitK == 4 || splitK == 8)) {
+        if (const TuneEntry *e = tune_lookup(xbits, M, N, K)) {
+            const TuneCfg &t = e->sk[splitK == 1 ? 0 : splitK == 2 ? 1 : splitK == 4 ? 2 : 3];
+            if (cfg_fits(t, M)) return LaunchCfg{ t.kind, t.nt, t.rt, t.wr, t.wk };
+        }
+    }
     size_t    tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
     if (N <= 16) {
         c.kind = 0;
         c.nt = 1;
         c.wr = 1;
-        // measured on MI355X: sharing the activation registers among four row tiles wins as soon as M/64 workgroups of four
-        // wavefronts cover about 60 % of the CUs; two row tiles need a full set of workgroups; otherwise one row tile
-        // per workgroup with as many wavefronts as there are K blocks to hand out.
-        if (tiles % 4 == 0 && (tiles / 4) * splitK * 100 >= (size_t)cus * 60) {
-            c.rt = 4;
-            c.wk = 4;
-        } else if (tiles % 2 == 0 && (tiles / 2) * splitK >= (size_t)cus) {
-            c.rt = 2;
-            c.wk = per_split > 8 ? (xbits == 5 ? 8 : 16) : per_split > 4 ? 8 : 4;
+        // Fitted to a sweep of every compiled shape over M in 2048..28672, K in 4096..28672, N in 1..16, both formats, on
+        // the MI355X.  What it encodes: about eight to eleven wavefronts per CU keep the memory system full; small
+        // workgroups (four wavefronts) balance better than large ones once there are several per CU; sharing the
+        // activation registers among row tiles (rt) pays in proportion to the batch, because every workgroup pulls the
+        // whole activation matrix through its CU's L1.
+        const double per_cu = (double)tiles * splitK / cus; // 16-row tiles per CU
+        if (N <= 4) {
+            if (per_cu < 1.5)        { c.rt = 1; c.wk = N <= 2 ? 16 : 8; }
+            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 8; }
+            else if (per_cu < 3.125) { c.rt = 1; c.wk = 4; }
+            else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
+            else                     { c.rt = 2; c.wk = 8; }
+        } else if (N <= 8) {
+            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
+            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 8; }
+            else if (per_cu < 3.125) { c.rt = 4; c.wk = 8; }
+            else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
+            else                     { c.rt = 4; c.wk = 4; }
         } else {
-            c.rt = 1;
-            c.wk = per_split > 8 ? 16 : per_split > 4 ? 8 : 4;
+            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
+            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 4; }
+            else                     { c.rt = 4; c.wk = 4; }
         }
+        while (c.rt > 1 && tiles % c.rt) c.rt /= 2;
+        const int cap = per_split > 8 ? 16 : per_split > 4 ? 8 : 4; // no more wavefronts than K blocks to hand out
+        if (c.wk > cap) c.wk = cap;
+        if (c.rt == 4 && c.wk == 16) c.wk = 8; // not compiled: 16 wavefronts leave too few registers for four row tiles
+        (void)xbits;
         return c;
     }
     c.kind = 1;
@@ -816,7 +878,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
     if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<XB, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
         FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
-        FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1)
+        FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1) FP6MI_CASE(4, 1, 4, 2) FP6MI_CASE(2, 1, 2, 4)
 #undef FP6MI_CASE
     }
     return FP6MI_ERR_SHAPE;
@@ -883,6 +945,18 @@ int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus)
 {
     if (M == 0 || N == 0 || K == 0 || num_cus <= 0) return 1;
     size_t units = (K + 255) / 256;
+    if (num_cus == 256) { // a measured neighbour knows better than any model: take its fastest split (3 % hysteresis towards fewer splits)
+        if (const TuneEntry *e = tune_lookup(6, M, N, K)) {
+            int      best_s = 0;
+            unsigned best_t = 0;
+            for (int i = 0; i < 4; i++) {
+                const TuneCfg &t = e->sk[i];
+                if (!cfg_fits(t, M) || (size_t)(1 << i) > units) continue;
+                if (best_s == 0 || (unsigned)t.t * 103u < best_t * 100u) { best_s = 1 << i; best_t = t.t; }
+            }
+            if (best_s) return best_s;
+        }
+    }
     if (N > 16) {
         size_t p = tile_k_parallelism(M, N, num_cus);
         size_t afford = (size_t)(0.5 * (double)K * 0.75 / (8.0 * (double)N));
@@ -938,6 +1012,17 @@ int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const vo
     LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
     return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, &c) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, &c);
+}
+
+int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, int *shape)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (!shape) return FP6MI_ERR_NULL;
+    if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
+    if (splitK < 1) return FP6MI_ERR_SPLITK;
+    LaunchCfg c = pick_cfg(E == 3 ? 6 : 5, M, N, K, splitK, 256);
+    shape[0] = c.kind, shape[1] = c.nt, shape[2] = c.rt, shape[3] = c.wr, shape[4] = c.wk;
+    return FP6MI_OK;
 }
 
 // ---- drop-in entry on REFERENCE-layout weights: native twins are made on first sight of a weight pointer and kept ----

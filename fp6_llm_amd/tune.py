@@ -1,0 +1,199 @@
+"""Launch-shape tuner of the FPx x FP16 GEMM.
+
+The engine chooses, per (format, M, N, K, splitK), one of its compiled kernel shapes.  A rule derived from first principles
+covers any shape; for the shapes of real models a measured table does better, the way BLAS libraries ship solution tables.
+This tool measures every candidate shape on the GPU it runs on and writes that table:
+
+    python -m fp6_llm_amd.tune sweep --format 6 --out fp6_llm_amd/tuning/fp6_mi355x.jsonl      # minutes of GPU time
+    python -m fp6_llm_amd.tune emit fp6_llm_amd/tuning/*.jsonl                                  # -> csrc/fp6mi_tuning.inc
+    python -m fp6_llm_amd.build
+
+Timing protocol: weights rotate through a pool of distinct buffers larger than the last-level cache, `iters` launches are
+captured into one HIP graph, one replay is timed with events; the best of `reps` such measurements counts.
+"""
+import argparse
+import glob
+import json
+import os
+import sys
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+INC_PATH = os.path.join(HERE, "csrc", "fp6mi_tuning.inc")
+
+# (kind, n_tiles, row_tiles, row_waves, k_waves); kind 0 = stream kernel (batch <= 16 per n_tile), 1 = tile kernel
+STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 4) for wk in (4, 8, 16) if (rt, wk) != (4, 16)]
+STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4)]                      # two 16-column tiles per workgroup, batches 17..32
+TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
+        (1, 8, 2, 8, 1)]
+SPLITS = (1, 2, 4, 8)
+
+# every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip); the candidates above are the ones that
+# ever came within 3 % of the best in exhaustive sweeps
+COMPILED_STREAM = [(0, nt, rt, 1, wk) for (nt, rt, wk) in
+                   [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 4, 4), (1, 4, 8), (2, 1, 4), (2, 1, 8), (2, 2, 4),
+                    (2, 2, 8), (4, 1, 4), (4, 1, 8), (4, 2, 4), (4, 2, 8)]]
+COMPILED_TILE = [(1,) + c for c in
+                 [(2, 1, 4, 4), (2, 2, 4, 4), (2, 2, 4, 2), (2, 2, 4, 1), (2, 4, 4, 1), (2, 4, 4, 2), (4, 2, 4, 2), (4, 2, 4, 1), (4, 4, 4, 1),
+                  (4, 4, 2, 1), (4, 4, 2, 2), (8, 2, 4, 1), (8, 2, 2, 1), (4, 2, 8, 1), (4, 2, 8, 2), (2, 2, 8, 1), (2, 2, 8, 2), (8, 2, 8, 1),
+                  (4, 1, 8, 2), (4, 1, 8, 1), (4, 1, 4, 2), (2, 1, 2, 4)]]
+
+GRID_M = [1024, 2048, 3072, 4096, 5120, 6144, 8192, 10240, 11008, 12288, 14336, 16384, 22016, 28672, 32768]
+GRID_K = [2048, 4096, 5120, 8192, 11008, 14336, 28672]
+GRID_N_SMALL = [1, 4, 8, 12, 16]
+GRID_N_LARGE = [24, 32, 48, 64, 96, 128, 256, 512]
+MAX_WEIGHTS = 28672 * 8192   # skip matrices beyond the largest layer of a 70B model
+
+
+def tile_rows(cfg):
+    kind, nt, rt, wr, wk = cfg
+    return 16 * rt * (wr if kind == 1 else 1)
+
+
+def candidates(OC, IC, BS):
+    if BS <= 16:
+        cfgs = STREAM_SMALL
+    else:
+        cfgs = [c for c in TILE if c[1] * 16 < 2 * BS + 16 or c[1] == 2]
+        if BS <= 32:
+            cfgs = cfgs + STREAM_WIDE
+    units = (IC + 255) // 256
+    for cfg in cfgs:
+        if OC % tile_rows(cfg):
+            continue
+        for sk in SPLITS:
+            if sk > units or (cfg[0] == 0 and sk > 1 and OC > 4096):   # the stream kernel splits K inside the workgroup already
+                continue
+            if sk > 1 and sk * 8 * BS > IC * 0.75:   # the FP32 partial sums would outweigh the weights themselves
+                continue
+            yield cfg, sk
+
+
+class Bench:
+    """Times one launch shape on one problem; keeps the weight pool of the current (format, OC, IC) alive between calls."""
+
+    def __init__(self, iters=30, reps=2, pool_bytes=1 << 30):
+        import torch
+
+        from . import _lib
+        self.torch, self.L = torch, _lib.lib()
+        self.iters, self.reps, self.pool_bytes = iters, reps, pool_bytes
+        self.dev = torch.device("cuda:0")
+        self.key = None
+
+    def _pool(self, E, M, OC, IC):
+        torch = self.torch
+        from . import native_bytes
+        if self.key != (E, M, OC, IC):
+            self.bufs = None
+            torch.cuda.empty_cache()
+            nb = native_bytes(E, M, OC, IC)
+            nbuf = max(2, min(48, self.pool_bytes // nb))
+            w0 = torch.randint(-2 ** 31, 2 ** 31 - 1, (nb // 4,), dtype=torch.int32)   # every bit pattern is a valid weight
+            self.bufs = [torch.roll(w0, 17 * i).to(self.dev) for i in range(nbuf)]
+            self.scales = (torch.rand(OC) * 0.009 + 0.001).half().to(self.dev)
+            self.key = (E, M, OC, IC)
+        return self.bufs, self.scales
+
+    def __call__(self, E, M, OC, IC, BS, cfg, sk):
+        torch = self.torch
+        bufs, scales = self._pool(E, M, OC, IC)
+        x = torch.randn(BS, IC).half().to(self.dev)
+        out = torch.empty(BS, OC, dtype=torch.float16, device=self.dev)
+        ws = torch.empty(sk * BS * OC, dtype=torch.float32, device=self.dev) if sk > 1 else None
+
+        def launch(i):
+            st = torch.cuda.current_stream().cuda_stream
+            return self.L.fp6mi_linear_native_cfg(E, M, st, bufs[i % len(bufs)].data_ptr(), scales.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                                  OC, BS, IC, ws.data_ptr() if ws is not None else None, sk, *cfg)
+        best = None
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            if launch(0) != 0:
+                return None
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(self.iters):
+                    launch(i)
+            graph.replay()
+            torch.cuda.synchronize()
+            for _ in range(self.reps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
+                graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                t = e0.elapsed_time(e1) * 1e3 / self.iters
+                best = t if best is None else min(best, t)
+        return best
+
+
+def sweep(args):
+    E, M = (3, 2) if args.format == 6 else (2, 2)
+    Ms = [int(v) for v in args.m.split(",")] if args.m else GRID_M
+    Ks = [int(v) for v in args.k.split(",")] if args.k else GRID_K
+    Ns = [int(v) for v in args.n.split(",")] if args.n else GRID_N_SMALL + GRID_N_LARGE
+    bench = Bench(args.iters, args.reps)
+    os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
+    with open(args.out, "a" if args.append else "w") as f:
+        for OC in Ms:
+            for IC in Ks:
+                if OC * IC > MAX_WEIGHTS:
+                    continue
+                for BS in Ns:
+                    best = {}
+                    for cfg, sk in candidates(OC, IC, BS):
+                        t = bench(E, M, OC, IC, BS, cfg, sk)
+                        if t is not None and (str(sk) not in best or t < best[str(sk)][1]):
+                            best[str(sk)] = [list(cfg), round(t, 3)]
+                    f.write(json.dumps({"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best}) + "\n")
+                    f.flush()
+                    print("e%dm%d %dx%d N=%d: " % (E, M, OC, IC, BS) + "  ".join("sk%s %s %.2f" % (k, "".join(map(str, v[0])), v[1]) for k, v in best.items()),
+                          flush=True)
+
+
+def emit(args):
+    rows = {}
+    for path in sorted(p for pat in args.files for p in glob.glob(pat)):
+        for line in open(path):
+            r = json.loads(line)
+            rows[(1 + r["E"] + r["M"], r["BS"], r["OC"], r["IC"])] = r   # later files override earlier ones
+    lines = ["// Measured launch shapes: generated by `python -m fp6_llm_amd.tune emit`; do not edit by hand.",
+             "// {bits, M/256, K/64, N, {best shape for splitK 1, 2, 4, 8: kind, n_tiles, row_tiles, row_waves, k_waves, time in 0.02 us}}"]
+    for (xb, BS, OC, IC) in sorted(rows):
+        r = rows[(xb, BS, OC, IC)]
+        cells = []
+        for sk in ("1", "2", "4", "8"):
+            if sk in r["best"]:
+                cfg, t = r["best"][sk]
+                cells.append("{%d,%d,%d,%d,%d,%d}" % (*cfg, min(65535, int(round(t / 0.02)))))
+            else:
+                cells.append("{255,0,0,0,0,0}")
+        lines.append("{%d,%d,%d,%d,{%s}}," % (xb, OC // 256, IC // 64, BS, ",".join(cells)))
+    with open(INC_PATH, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    print("%d entries -> %s" % (len(rows), INC_PATH))
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
+    sub = ap.add_subparsers(dest="cmd", required=True)
+    s = sub.add_parser("sweep")
+    s.add_argument("--format", type=int, choices=(5, 6), default=6)
+    s.add_argument("--out", required=True)
+    s.add_argument("--append", action="store_true")
+    s.add_argument("--m", default="")
+    s.add_argument("--k", default="")
+    s.add_argument("--n", default="")
+    s.add_argument("--iters", type=int, default=30)
+    s.add_argument("--reps", type=int, default=2)
+    s.set_defaults(fn=sweep)
+    e = sub.add_parser("emit")
+    e.add_argument("files", nargs="+")
+    e.set_defaults(fn=emit)
+    args = ap.parse_args(argv)
+    args.fn(args)
+
+
+if __name__ == "__main__":
+    sys.exit(main())

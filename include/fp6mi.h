@@ -99,6 +99,13 @@ int fp6mi_linear_native_cfg(int E, int Mbits, void *stream, const void *W_native
                             const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK,
                             int kind, int n_tiles, int row_tiles, int row_waves, int k_waves);
 
+/* Which kernel shape fp6mi_linear_native would launch for this problem: shape[0..4] = kind, n_tiles, row_tiles,
+ * row_waves, k_waves, with the meaning they have in fp6mi_linear_native_cfg.  Pure host code, no GPU needed.  The
+ * choice comes from a table measured on the MI355X (python -m fp6_llm_amd.tune) where the problem is near a measured
+ * one, else from a rule; it plays the part of the reference's compile-time TilingConfig dispatch
+ * (fp6_llm/csrc/fp6_linear.cu:61-81). */
+int fp6mi_query_launch(int E, int Mbits, size_t M, size_t N, size_t K, int splitK, int *shape);
+
 /* Device-side conversion reference layout -> native layout (both device pointers), run once per weight matrix. */
 int fp6mi_relayout_ref_to_native_gpu(int E, int Mbits, void *stream, void *native_dev, const void *packed_ref_dev,
                                      size_t M, size_t K);

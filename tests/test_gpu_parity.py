@@ -130,12 +130,7 @@ def test_split_k(E, M, splitK):
     check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "splitK=%d" % splitK)
 
 
-STREAM_SHAPES = [(0, 1, 1, 1, 4), (0, 1, 1, 1, 8), (0, 1, 1, 1, 16), (0, 1, 2, 1, 4), (0, 1, 2, 1, 8), (0, 1, 2, 1, 16), (0, 1, 4, 1, 4),
-                 (0, 1, 4, 1, 8), (0, 2, 1, 1, 4), (0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 2, 1, 8), (0, 4, 1, 1, 4), (0, 4, 1, 1, 8),
-                 (0, 4, 2, 1, 4), (0, 4, 2, 1, 8)]
-TILE_SHAPES = [(1, 2, 1, 4, 4), (1, 2, 2, 4, 4), (1, 2, 2, 4, 2), (1, 2, 2, 4, 1), (1, 2, 4, 4, 1), (1, 2, 4, 4, 2), (1, 4, 2, 4, 2),
-               (1, 4, 2, 4, 1), (1, 4, 4, 4, 1), (1, 4, 4, 2, 1), (1, 4, 4, 2, 2), (1, 8, 2, 4, 1), (1, 8, 2, 2, 1), (1, 4, 2, 8, 1), (1, 4, 2, 8, 2), (1, 2, 2, 8, 1),
-               (1, 2, 2, 8, 2), (1, 8, 2, 8, 1), (1, 4, 1, 8, 2), (1, 4, 1, 8, 1)]
+from fp6_llm_amd.tune import COMPILED_STREAM as STREAM_SHAPES, COMPILED_TILE as TILE_SHAPES  # noqa: E402
 
 
 @pytest.mark.parametrize("E,M", FORMATS)

@@ -183,13 +183,60 @@ def test_reference_heuristic_is_kept_verbatim():
 def test_mi355x_heuristic_prefers_no_split_when_rows_fill_the_chip():
     for (M, N, K) in [(4096, 8, 4096), (11008, 8, 4096), (8192, 16, 8192), (28672, 8, 8192), (8192, 512, 8192)]:
         assert fp6.heuristic_splitk_mi355x(M, N, K) == 1
-    # batches above 16 use 128-row tiles: K is cut until about four wavefronts per CU exist, partial-sum traffic permitting
-    assert fp6.heuristic_splitk_mi355x(8192, 32, 8192) == 8
-    assert fp6.heuristic_splitk_mi355x(28672, 32, 8192) == 2
-    assert fp6.heuristic_splitk_mi355x(8192, 64, 8192) == 4
+    # batches above 16 tile the rows in blocks of 64..256: K is cut to make up the missing parallelism, by a power of two
+    # of at most 8 and never into more pieces than there are 256-column K blocks
+    for (M, N, K) in [(8192, 32, 8192), (28672, 32, 8192), (8192, 64, 8192), (4096, 32, 11008), (10240, 32, 8192), (4096, 128, 512)]:
+        s = fp6.heuristic_splitk_mi355x(M, N, K)
+        assert s in (1, 2, 4, 8) and s <= (K + 255) // 256, (M, N, K, s)
+    assert fp6.heuristic_splitk_mi355x(8192, 32, 8192) > 1          # 64 row blocks alone leave three quarters of the CUs idle
     s = fp6.heuristic_splitk_mi355x(256, 8, 28672)      # 16 row tiles cannot occupy 256 CUs: splitting K pays
     assert 2 <= s <= 64
     assert fp6.heuristic_splitk_mi355x(256, 1, 1024) == 1  # too little work to pay for a second launch
+
+
+def test_rule_based_heuristic_for_other_cu_counts():
+    """With a CU count that has no measured table the cost rules decide; known answers of those rules for a 304-CU part."""
+    assert fp6.heuristic_splitk_mi355x(4096, 8, 4096, 304) == 1
+    assert fp6.heuristic_splitk_mi355x(8192, 512, 8192, 304) == 1
+    for (M, N, K) in [(8192, 32, 8192), (28672, 32, 8192), (8192, 64, 8192)]:
+        s = fp6.heuristic_splitk_mi355x(M, N, K, 304)
+        assert s in (1, 2, 4, 8)
+    assert fp6.heuristic_splitk_mi355x(8192, 32, 8192, 304) >= fp6.heuristic_splitk_mi355x(28672, 32, 8192, 304)
+
+
+def test_compiled_launch_shape_lists_match_the_kernel_source():
+    from fp6_llm_amd import tune
+    src = open(os.path.join(os.path.dirname(fp6.__file__), "csrc", "fp6mi_gemm.hip")).read()
+    stream = {(0, int(a), int(b), 1, int(c)) for a, b, c in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+)\)", src)}
+    tile = {(1, int(a), int(b), int(c), int(d)) for a, b, c, d in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+), (\d+)\)", src)}
+    assert stream == set(tune.COMPILED_STREAM) and tile == set(tune.COMPILED_TILE)
+    assert set(tune.STREAM_SMALL + tune.STREAM_WIDE) <= stream and set(tune.TILE) <= tile
+
+
+def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it():
+    from fp6_llm_amd import tune
+    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE)
+    inc = open(tune.INC_PATH).read()
+    entries = re.findall(r"^\{(\d+),(\d+),(\d+),(\d+),\{(.*)\}\},$", inc, flags=re.M)
+    L = _lib.lib()
+    shape = (ctypes.c_int * 5)()
+    for xb, m256, k64, n, cells in entries:
+        E = 3 if int(xb) == 6 else 2
+        OC, IC, BS = int(m256) * 256, int(k64) * 64, int(n)
+        for i, cell in enumerate(re.findall(r"\{([\d,]+)\}", cells)):
+            v = tuple(int(t) for t in cell.split(","))
+            if v[0] == 255:
+                continue
+            assert v[:5] in compiled, (xb, OC, IC, BS, v)
+            assert OC % tune.tile_rows(v[:5]) == 0
+            assert L.fp6mi_query_launch(E, 2, OC, BS, IC, 1 << i, shape) == 0
+            assert tuple(shape) == v[:5], (xb, OC, IC, BS, 1 << i, tuple(shape), v)
+    # any legal problem gets a compiled shape that divides its rows, measured neighbour or not
+    for (OC, IC, BS, sk) in [(256, 64, 1, 1), (768, 1088, 3, 2), (4352, 4160, 8, 1), (9984, 3008, 40, 3), (65536, 16384, 700, 1), (512, 64, 17, 1)]:
+        for E in (3, 2):
+            assert L.fp6mi_query_launch(E, 2, OC, BS, IC, sk, shape) == 0
+            assert tuple(shape) in compiled and OC % tune.tile_rows(tuple(shape)) == 0, (OC, IC, BS, sk, tuple(shape))
+    assert L.fp6mi_query_launch(3, 2, 100, 1, 64, 1, shape) == -2 and L.fp6mi_query_launch(4, 3, 256, 1, 64, 1, shape) == -1
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
