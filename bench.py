@@ -7,7 +7,9 @@ A step is one GEMM of the workload (default: the headline one, FP6_e3m2 4096x409
 heuristic).  Weights are synthetic, already resident in HBM, and ROTATE through a pool of distinct buffers larger than the
 256 MB last-level cache, so every step streams its weights from HBM like consecutive layers of a model would ("cold");
 the same-buffer ("warm") figure is reported beside it.  The K steps are captured once into a HIP graph and replayed inside
-the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 us kernel.
+the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 us kernel.  The graph is first replayed
+untimed for ~60 ms (right after an idle spell the GPU runs 10-15 % slow), then five replays are timed one by one, each
+exactly K steps between two synchronizations, and the median is reported; the FP16 baseline is timed the same way.
 
 Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth figure the reference's design is judged
 on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
@@ -99,6 +101,38 @@ class Problem:
         fp6.linear_forward_native(self.E, self.M, self.x, w, self.scales, self.OC, self.splitK, out=self.out, workspace=self.ws)
 
 
+CLOCK_WARMUP_MS = 60.0   # untimed graph replays before the timed ones: the first replays after an idle spell run 10-15 % slow
+TIMED_REPLAYS = 5        # each times exactly `steps` steps between two synchronizations; the median is reported
+
+
+def _timed_replays(graph, steps):
+    """Replays the captured K-step graph untimed until the clocks have settled, then times TIMED_REPLAYS replays one by one.
+    Returns (median wall seconds, median HIP-event milliseconds) of one replay."""
+    import torch
+
+    spent, n = 0.0, 0
+    while n < 2 or (spent < CLOCK_WARMUP_MS and n < 50):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        spent += e0.elapsed_time(e1)
+        n += 1
+    walls, evs = [], []
+    for _ in range(TIMED_REPLAYS):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        walls.append(time.perf_counter() - t0)
+        evs.append(e0.elapsed_time(e1))
+    return sorted(walls)[len(walls) // 2], sorted(evs)[len(evs) // 2]
+
+
 def time_steps(prob, steps, warmup, cold):
     """Returns (wall seconds between the two synchronizations, HIP-event milliseconds on the launch stream)."""
     import torch
@@ -112,16 +146,7 @@ def time_steps(prob, steps, warmup, cold):
         with torch.cuda.graph(graph, stream=stream):
             for i in range(steps):
                 prob.step(warmup + i, cold)
-        graph.replay()  # untimed: first replay uploads the graph
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        t0 = time.perf_counter()
-        e0.record()
-        graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-        t1 = time.perf_counter()
-    return t1 - t0, e0.elapsed_time(e1)
+        return _timed_replays(graph, steps)
 
 
 def read_floor_us(prob, steps, warmup):
@@ -154,14 +179,8 @@ def read_floor_us(prob, steps, warmup):
         with torch.cuda.graph(graph, stream=stream):
             for i in range(steps):
                 step(warmup + i)
-        graph.replay()
-        torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        e0.record()
-        graph.replay()
-        e1.record()
-        torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / steps
+        _, ev_ms = _timed_replays(graph, steps)
+    return ev_ms * 1e3 / steps
 
 
 def fp16_baseline_us(prob, steps, warmup):
@@ -180,25 +199,22 @@ def fp16_baseline_us(prob, steps, warmup):
     with torch.cuda.stream(stream):
         torch.nn.functional.linear(prob.x, ws[0])
         torch.cuda.synchronize()
-        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         try:
             graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(graph, stream=stream):
                 for i in range(steps):
                     torch.nn.functional.linear(prob.x, ws[i % nbuf])
-            graph.replay()
-            torch.cuda.synchronize()
-            e0.record()
-            graph.replay()
-            e1.record()
+            _, ev_ms = _timed_replays(graph, steps)
         except RuntimeError:  # the BLAS library refused capture: time plain launches instead
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
             torch.cuda.synchronize()
             e0.record()
             for i in range(steps):
                 torch.nn.functional.linear(prob.x, ws[i % nbuf])
             e1.record()
-        torch.cuda.synchronize()
-    return e0.elapsed_time(e1) * 1e3 / steps
+            torch.cuda.synchronize()
+            ev_ms = e0.elapsed_time(e1)
+    return ev_ms * 1e3 / steps
 
 
 def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
