@@ -6,7 +6,7 @@
 A step is one GEMM of the workload (default: the headline one, FP6_e3m2 4096x4096, batch 8, split-K from the engine's
 heuristic).  Weights are synthetic, already resident in HBM, and ROTATE through a pool of distinct buffers larger than the
 256 MB last-level cache, so every step streams its weights from HBM like consecutive layers of a model would ("cold");
-the same-buffer ("warm") figure is reported beside it.  The K steps are captured once into a HIP graph and replayed inside
+--warm (and --sweep) add the same-buffer figure.  The K steps are captured once into a HIP graph and replayed inside
 the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 us kernel.  The graph is first replayed
 untimed for ~60 ms (right after an idle spell the GPU runs 10-15 % slow), then five replays are timed one by one, each
 exactly K steps between two synchronizations, and the median is reported; the FP16 baseline is timed the same way.
@@ -53,10 +53,11 @@ HEADLINE = "fp6_4096x4096_bs8"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
 # for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
-    "fp6_4096x4096_bs8": 13241840,
-    "fp6_8192x8192_bs8": 51572091,
-    "fp6_28672x8192_bs32": 187771045,   # GEMM kernel only; its split-K reduction kernel is a separate dispatch
-    "fp6_8192x8192_bs512": 126075242,
+    "fp6_4096x4096_bs8": 13244911,
+    "fp6_8192x8192_bs8": 51570043,
+    "fp5_8192x8192_bs8": 43196662,
+    "fp6_28672x8192_bs32": 182255785,
+    "fp6_8192x8192_bs512": 125981259,
 }
 
 
@@ -248,21 +249,23 @@ def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
     }
 
 
-def run_workload(name, steps, warmup, device, with_fp16=True):
+def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True):
     E, M, OC, IC, BS = WORKLOADS[name]
     prob = Problem(E, M, OC, IC, BS, device)
     wall_s, ev_ms = time_steps(prob, steps, warmup, cold=True)
-    _, ev_ms_warm = time_steps(prob, steps, warmup, cold=False)
     us = ev_ms * 1e3 / steps
-    us_warm = ev_ms_warm * 1e3 / steps
+    us_warm = time_steps(prob, steps, warmup, cold=False)[1] * 1e3 / steps if with_warm else float("nan")
     wb = weight_bytes(E, M, OC, IC)
     flops = 2.0 * OC * IC * BS
     res = {
-        "workload": name, "us_per_gemm": round(us, 3), "us_per_gemm_wall": round(wall_s * 1e6 / steps, 3), "us_per_gemm_warm": round(us_warm, 3),
-        "weight_GBps": round(wb / us / 1e3, 1), "weight_GBps_warm": round(wb / us_warm / 1e3, 1), "tflops": round(flops / us / 1e6, 2),
+        "workload": name, "us_per_gemm": round(us, 3), "us_per_gemm_wall": round(wall_s * 1e6 / steps, 3),
+        "weight_GBps": round(wb / us / 1e3, 1), "tflops": round(flops / us / 1e6, 2),
         "hbm_frac": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
         "splitK": prob.splitK, "weight_buffers": prob.nbuf, "weight_bytes": wb, "algorithmic_bytes": algorithmic_bytes(E, M, OC, IC, BS),
     }
+    if with_warm:   # same weight buffer every step: served by the last-level cache when it fits
+        res["us_per_gemm_warm"] = round(us_warm, 3)
+        res["weight_GBps_warm"] = round(wb / us_warm / 1e3, 1)
     floor = read_floor_us(prob, steps, warmup)
     if floor is not None:
         res["read_floor_us"] = round(floor, 3)               # a kernel that only reads these weight buffers once
@@ -286,6 +289,7 @@ def main():
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration (writes gpurun_out/bench_sweep.jsonl)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--warm", action="store_true", help="also time the workload with the same weight buffer every step (cache-resident weights)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by")
     args = ap.parse_args()
@@ -306,7 +310,7 @@ def main():
         for _ in range(10):
             dst.copy_(src)
         torch.cuda.synchronize()
-    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy)
+    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy, with_warm=args.warm)
     E, M, OC, IC, BS = WORKLOADS[args.workload]
     line = {
         "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",
