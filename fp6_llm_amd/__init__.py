@@ -210,6 +210,9 @@ def _workspace(device, stream, nbytes):
     return ws
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the current stream's handle without building a Stream object
+
+
 def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, splitK=1, out=None, workspace=None):
     """out[B, OC] = in_feats[B, IC] @ dequant(W)^T with W in the native layout.  Enqueued on the current stream."""
     _bits(EXPONENT, MANTISSA)
@@ -225,29 +228,41 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
     B, IC = in_feats.shape
     if OC % 256 != 0 or IC % 64 != 0 or B < 1:
         raise ValueError("need OC %% 256 == 0, IC %% 64 == 0, B >= 1 (got OC=%d IC=%d B=%d)" % (OC, IC, B))
-    if native_weight.numel() * native_weight.element_size() != native_bytes(EXPONENT, MANTISSA, OC, IC):
+    # same value as fp6mi_native_bytes, computed here: this function is on the per-token path and a 5 us kernel deserves a
+    # wrapper that costs less than it does
+    if native_weight.numel() * native_weight.element_size() != (OC // 16) * ((IC + 255) // 256) * (3072 if EXPONENT == 3 else 2560):
         raise ValueError("native_weight has the wrong size for OC=%d IC=%d" % (OC, IC))
-    if int(splitK) < 1:
-        raise ValueError("splitK must be >= 1")
     splitK = int(splitK)
-    x = in_feats.contiguous()
-    sc = scales.contiguous()
+    if splitK < 1:
+        raise ValueError("splitK must be >= 1")
+    x = in_feats if in_feats.is_contiguous() else in_feats.contiguous()
+    sc = scales if scales.is_contiguous() else scales.contiguous()
     if out is None:
         out = torch.empty((B, OC), dtype=torch.float16, device=dev)
     elif out.shape != (B, OC) or out.dtype != torch.float16 or not out.is_contiguous() or out.device != dev:
         raise ValueError("out must be a contiguous float16 [B, OC] tensor on the same GPU")
-    with torch.cuda.device(dev):
-        stream = torch.cuda.current_stream().cuda_stream
+    L = _lib.lib()
+    switch = dev.index is not None and dev.index != torch.cuda.current_device()
+    if switch:
+        prev = torch.cuda.current_device()
+        torch.cuda.set_device(dev)
+    try:
+        stream = _raw_stream(dev.index) if _raw_stream is not None and dev.index is not None else torch.cuda.current_stream().cuda_stream
         ws_ptr = None
         if splitK > 1:
-            need = _lib.lib().fp6mi_workspace_bytes(OC, B, splitK)
+            need = 4 * splitK * OC * B
             if workspace is None:
                 workspace = _workspace(dev, stream, need)
             elif workspace.dtype != torch.float32 or workspace.numel() * 4 < need or workspace.device != dev:
                 raise ValueError("workspace must be a float32 GPU tensor with at least splitK*B*OC elements")
             ws_ptr = workspace.data_ptr()
-        _lib.check(_lib.lib().fp6mi_linear_native(EXPONENT, MANTISSA, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(),
-                                                  out.data_ptr(), OC, B, IC, ws_ptr, splitK), "fp6mi_linear_native")
+        rc = L.fp6mi_linear_native(EXPONENT, MANTISSA, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(),
+                                   out.data_ptr(), OC, B, IC, ws_ptr, splitK)
+    finally:
+        if switch:
+            torch.cuda.set_device(prev)
+    if rc != 0:
+        _lib.check(rc, "fp6mi_linear_native")
     return out
 
 

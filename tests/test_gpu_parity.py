@@ -289,6 +289,19 @@ def test_module_forward():
         check_close(y.reshape(10, 512).cpu().numpy(), ref, "module e%dm%d" % (E, M))
 
 
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_command_line_harness(E, M):
+    """The counterpart of the reference's tests/python/kernel_test_fpx.py: same flags, same printed quantities."""
+    import io
+    from fp6_llm_amd import kernel_test
+    buf = io.StringIO()
+    res = kernel_test.run(512, 1280, 9, splitK=0, EXP=E, MAN=M, repeat=5, warmup=2, out=buf)
+    assert res["max_rel_err_vs_fp32"] <= 1e-2 and res["mean_err_vs_fp16_gemm"] <= 2e-3
+    assert res["fpx_ms"] > 0 and res["speedup"] > 0 and "speed-up" in buf.getvalue()
+    res = kernel_test.run(256, 2048, 40, splitK=2, EXP=E, MAN=M, repeat=3, warmup=1, out=buf)
+    assert res["splitK"] == 2 and res["max_rel_err_vs_fp32"] <= 1e-2
+
+
 # ------------------------------------------------------------------------------------------------ device-side quantizer
 def _awkward_weights(seed, OC, IC, dtype):
     """Gaussian weights with the cases a quantizer gets wrong: an all-zero row, a row of tiny values whose scale rounds to
