@@ -24,6 +24,7 @@ class FPxLinear(torch.nn.Module):
         self.in_features, self.out_features = in_features, out_features
         self.exponent, self.mantissa = exponent, mantissa
         self.split_k = split_k
+        self._split_cache = {}
         self.register_buffer("weight_native", torch.zeros(native_bytes(exponent, mantissa, out_features, in_features) // 4, dtype=torch.int32))
         self.register_buffer("scales", torch.ones(out_features, dtype=torch.float16))
         self.register_buffer("bias", bias)
@@ -88,7 +89,11 @@ class FPxLinear(torch.nn.Module):
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype != torch.float16:
             x2 = x2.half()
-        sk = self.split_k or heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS)
+        sk = self.split_k
+        if not sk:   # the heuristic's answer per batch size is remembered: the layer is called once per token
+            sk = self._split_cache.get(x2.shape[0])
+            if sk is None:
+                sk = self._split_cache[x2.shape[0]] = heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS)
         y = linear_forward_native(self.exponent, self.mantissa, x2, self.weight_native, self.scales, self.out_features, sk)
         if self.bias is not None:
             y = y + self.bias
