@@ -184,38 +184,106 @@ def read_floor_us(prob, steps, warmup):
     return ev_ms * 1e3 / steps
 
 
+class _RocblasFp16:
+    """rocblas_gemm_ex (FP16 in/out, FP32 accumulation) through ctypes: the second FP16 library path on this stack, which
+    for some shapes picks a faster kernel than torch's F.linear and for others a much slower one."""
+
+    def __init__(self):
+        import ctypes
+        self.ct = ctypes
+        self.lib = ctypes.CDLL("librocblas.so")
+        self.handle = ctypes.c_void_p()
+        if self.lib.rocblas_create_handle(ctypes.byref(self.handle)) != 0:
+            raise RuntimeError("rocblas_create_handle failed")
+        vp, ci, u32 = ctypes.c_void_p, ctypes.c_int, ctypes.c_uint32
+        self.lib.rocblas_set_stream.argtypes = [vp, vp]
+        self.lib.rocblas_gemm_ex.argtypes = [vp, ci, ci, ci, ci, ci, vp, vp, ci, ci, vp, ci, ci, vp, vp, ci, ci, vp, ci, ci, ci, ci, ctypes.c_int32, u32]
+        self.alpha, self.beta = ctypes.c_float(1.0), ctypes.c_float(0.0)
+
+    def linear(self, x, w, out, stream):
+        """out[B, OC] = x[B, IC] @ w[OC, IC]^T; column-major view: C[OC x B] = op_T(w as IC x OC) * (x as IC x B)."""
+        ct = self.ct
+        B, IC = x.shape
+        OC = w.shape[0]
+        self.lib.rocblas_set_stream(self.handle, stream)
+        rc = self.lib.rocblas_gemm_ex(self.handle, 112, 111, OC, B, IC, ct.addressof(self.alpha), w.data_ptr(), 150, IC, x.data_ptr(), 150, IC,
+                                      ct.addressof(self.beta), out.data_ptr(), 150, OC, out.data_ptr(), 150, OC, 151, 0, 0, 0)
+        if rc != 0:
+            raise RuntimeError("rocblas_gemm_ex failed with status %d" % rc)
+
+
+def _time_fp16(fn, steps, warmup):
+    import torch
+
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        fn(0)
+        torch.cuda.synchronize()
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    fn(i)
+            _, ev_ms = _timed_replays(graph, steps)
+        except RuntimeError:  # the BLAS library refused capture: time plain launches instead
+            torch.cuda.synchronize()
+            for i in range(3 * steps):   # untimed, to settle the clocks
+                fn(i)
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            torch.cuda.synchronize()
+            e0.record()
+            for i in range(steps):
+                fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            ev_ms = e0.elapsed_time(e1)
+    return ev_ms * 1e3 / steps
+
+
 def fp16_baseline_us(prob, steps, warmup):
-    """FP16 GEMM of the same shape on the same GPU (torch F.linear = hipBLASLt/rocBLAS), weights rotating the same way:
-    the counterpart of the reference's cuBLAS baseline (tests/python/kernel_test_fp6.py:45-62)."""
+    """FP16 GEMM of the same shape on the same GPU, weights rotating the same way: the counterpart of the reference's cuBLAS
+    baseline (tests/python/kernel_test_fp6.py:45-62, tests/cpp/kernel_test_fpx.cu:80-103).  Two library paths are timed,
+    torch F.linear (hipBLASLt) and rocblas_gemm_ex; returns (the faster one, {path: us})."""
     import torch
 
     dev = prob.x.device
     nb = prob.OC * prob.IC * 2
     nbuf = int(max(2, min(64, POOL_BYTES // nb)))
     ws = [torch.randn(prob.OC, prob.IC, dtype=torch.float16, device=dev) for _ in range(nbuf)]
-    for i in range(warmup):
-        torch.nn.functional.linear(prob.x, ws[i % nbuf])
-    torch.cuda.synchronize()
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        torch.nn.functional.linear(prob.x, ws[0])
+    out = torch.empty(prob.BS, prob.OC, dtype=torch.float16, device=dev)
+    res = {"torch_F_linear": _time_fp16(lambda i: torch.nn.functional.linear(prob.x, ws[i % nbuf]), steps, warmup)}
+    try:
+        rb = _RocblasFp16()
+        # same answer as F.linear before it is trusted as a baseline
+        rb.linear(prob.x, ws[0], out, torch.cuda.current_stream().cuda_stream)
         torch.cuda.synchronize()
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for i in range(steps):
-                    torch.nn.functional.linear(prob.x, ws[i % nbuf])
-            _, ev_ms = _timed_replays(graph, steps)
-        except RuntimeError:  # the BLAS library refused capture: time plain launches instead
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for i in range(steps):
-                torch.nn.functional.linear(prob.x, ws[i % nbuf])
-            e1.record()
-            torch.cuda.synchronize()
-            ev_ms = e0.elapsed_time(e1)
-    return ev_ms * 1e3 / steps
+        ref = torch.nn.functional.linear(prob.x, ws[0])
+        if torch.allclose(out.float(), ref.float(), rtol=2e-2, atol=2e-2 * float(ref.float().abs().mean())):
+            res["rocblas_gemm_ex"] = _time_fp16(lambda i: rb.linear(prob.x, ws[i % nbuf], out, torch.cuda.current_stream().cuda_stream), steps, warmup)
+    except (OSError, RuntimeError, AttributeError):
+        pass
+    return min(res.values()), res
+
+
+def fp16_system_blas_us(OC, IC, BS, steps):
+    """The same FP16 GEMM through the SYSTEM's rocBLAS/hipBLASLt, in a process of its own (torch bundles older copies of
+    those libraries, and the newer ones pick a faster kernel for some shapes): the C++ driver's `fp16` mode, eager
+    launches back to back on one stream, weights rotating through 1 GiB.  None if the driver is not built."""
+    import re
+    import subprocess
+
+    exe = os.path.join(ROOT, "fp6_llm_amd", "kernel_bench")
+    if not os.path.exists(exe):
+        return None
+    try:
+        res = subprocess.run([exe, "fp16", str(OC), str(IC), str(BS), str(steps), "20"], capture_output=True, text=True, timeout=300)
+    except (OSError, subprocess.SubprocessError):
+        return None
+    m = re.search(r": ([0-9.]+) us/GEMM", res.stdout)
+    return float(m.group(1)) if res.returncode == 0 and m else None
 
 
 def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
@@ -249,7 +317,7 @@ def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
     }
 
 
-def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True):
+def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True, with_system_blas=True):
     E, M, OC, IC, BS = WORKLOADS[name]
     prob = Problem(E, M, OC, IC, BS, device)
     wall_s, ev_ms = time_steps(prob, steps, warmup, cold=True)
@@ -275,8 +343,16 @@ def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True):
         del prob.weights[2:]
         import torch
         torch.cuda.empty_cache()
-        f16 = fp16_baseline_us(prob, min(steps, 200), min(warmup, 10))
-        res["fp16_gemm_us"] = round(f16, 3)
+        f16, paths = fp16_baseline_us(prob, min(steps, 200), min(warmup, 10))
+        if with_system_blas:
+            del prob
+            torch.cuda.empty_cache()
+            ext = fp16_system_blas_us(OC, IC, BS, min(steps, 500))
+            if ext is not None:
+                paths["system_rocblas_own_process"] = ext
+                f16 = min(f16, ext)
+        res["fp16_gemm_us"] = round(f16, 3)             # the fastest of the FP16 library paths
+        res["fp16_gemm_us_by_path"] = {k: round(v, 3) for k, v in paths.items()}
         res["speedup_vs_fp16"] = round(f16 / us, 3)
     return res, wall_s
 
@@ -288,7 +364,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
     ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration (writes gpurun_out/bench_sweep.jsonl)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-cpu-baseline", action="store_true",
+                    help="skip the legs that run outside this process's GPU stream: the CPU path and the system-BLAS FP16 baseline (a child process)")
     ap.add_argument("--warm", action="store_true", help="also time the workload with the same weight buffer every step (cache-resident weights)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by")
@@ -310,7 +387,8 @@ def main():
         for _ in range(10):
             dst.copy_(src)
         torch.cuda.synchronize()
-    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy, with_warm=args.warm)
+    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy, with_warm=args.warm,
+                               with_system_blas=not args.no_cpu_baseline)
     E, M, OC, IC, BS = WORKLOADS[args.workload]
     line = {
         "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",
