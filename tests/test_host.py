@@ -320,3 +320,18 @@ def test_e2m2_code_read_as_e3m2_is_a_quarter_of_its_value():
     for code in range(32):
         field = (code & 15) | ((code >> 4) << 5)
         assert v6[field] * 4.0 == v5[code] and np.signbit(v6[field]) == np.signbit(v5[code])
+
+
+def test_bench_refuses_more_than_one_gpu_and_lists_the_benchmark_configurations():
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    res = subprocess.run([sys.executable, os.path.join(root, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0 and "ONE GPU" in res.stderr
+    sys.path.insert(0, root)
+    import bench
+    assert bench.WORKLOADS[bench.HEADLINE] == (3, 2, 4096, 4096, 8)
+    # every shape of the five benchmark configurations is a workload: 4096^2 at 1/8/16, the two 7B MLP shapes at 8/32, the three
+    # 70B shapes at 32, and 8192^2 at ten batch sizes in both formats
+    assert len(bench.WORKLOADS) == 3 + 4 + 3 + 20
+    assert bench.weight_bytes(3, 2, 4096, 4096) == 12582912 and bench.algorithmic_bytes(3, 2, 4096, 4096, 8) == 12722176
