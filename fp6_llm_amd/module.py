@@ -7,7 +7,7 @@ import numpy as np
 import torch
 
 from . import quant
-from . import (MI355X_CUS, heuristic_splitk_mi355x, linear_forward_native, native_bytes, to_native,
+from . import (MI355X_CUS, heuristic_splitk_mi355x, linear_forward_native, native_bytes, to_native, weight_dequant_native_cuda,
                weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu, weight_quantize_native_cuda)
 
 _MAGIC = b"FP6MI\x00\x01\x00"   # name, NUL, layout version 1, reserved
@@ -17,8 +17,13 @@ class FPxLinear(torch.nn.Module):
     """y = x @ dequant(W)^T (+ bias) with W held in the native gfx950 layout.  Weights are buffers, not parameters:
     the layer is inference-only, like the kernels."""
 
-    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None):
+    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None, dequant_above=None):
+        """dequant_above: batch size from which forward() dequantizes the weights to a temporary fp16 matrix on the GPU and calls
+        the FP16 library GEMM instead (prefill).  The mixed-input kernel wins while the GEMM is bound by weight bytes; from a
+        couple of thousand rows the FP16 library runs 1.3-1.4 PFLOP/s against its 0.9-1.0 (measured at 8192 x 8192), which
+        pays for the dequantization pass.  None (default) never does: the temporary costs 2 bytes per weight."""
         super().__init__()
+        self.dequant_above = dequant_above
         if out_features % 256 or in_features % 64:
             raise ValueError("FPxLinear needs out_features %% 256 == 0 and in_features %% 64 == 0")
         self.in_features, self.out_features = in_features, out_features
@@ -89,6 +94,13 @@ class FPxLinear(torch.nn.Module):
         x2 = x.reshape(-1, self.in_features)
         if x2.dtype != torch.float16:
             x2 = x2.half()
+        if self.dequant_above is not None and x2.shape[0] >= self.dequant_above:
+            w16 = weight_dequant_native_cuda(self.exponent, self.mantissa, self.weight_native, self.scales, self.out_features, self.in_features)
+            y = torch.nn.functional.linear(x2, w16)
+            del w16
+            if self.bias is not None:
+                y = y + self.bias
+            return y.reshape(*lead, self.out_features)
         sk = self.split_k
         if not sk:   # the heuristic's answer per batch size is remembered: the layer is called once per token
             sk = self._split_cache.get(x2.shape[0])

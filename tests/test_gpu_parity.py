@@ -343,6 +343,22 @@ def test_device_quantizer_rejects_bad_arguments():
         fp6.weight_quantize_native_cuda(3, 2, torch.zeros(256, 128, dtype=torch.float16))
 
 
+def test_module_prefill_route_dequantizes_and_matches():
+    from fp6_llm_amd import module
+    w = torch.from_numpy(synth.normal(53, (256, 512))).half()
+    for (E, M) in FORMATS:
+        layer = module.FPxLinear.from_float(w, E, M).to(DEV)
+        layer.dequant_above = 64
+        x = torch.from_numpy(synth.activations(54, 100, 512)).to(DEV)
+        y_lib = layer(x)                       # 100 rows >= 64: dequantize + FP16 library GEMM
+        layer.dequant_above = None
+        y_fpx = layer(x)                       # the mixed-input kernel
+        codes, scales = quant.quantize_rowwise(w.float().numpy(), E, M)
+        ref = oracle.gemm_f64(oracle.dequant(quant.pack_raw(codes, E, M), scales, E, M), x.cpu().numpy())
+        check_close(y_lib.cpu().numpy(), ref, "prefill route e%dm%d" % (E, M))
+        check_close(y_fpx.cpu().numpy(), ref, "kernel route e%dm%d" % (E, M))
+
+
 def test_module_from_float_on_device_equals_host_path():
     from fp6_llm_amd import module
     w = torch.from_numpy(synth.normal(51, (512, 1024))).half()
