@@ -41,7 +41,7 @@ COMPILED_TILE = [(1,) + c for c in
 GRID_M = [1024, 2048, 3072, 4096, 5120, 6144, 8192, 10240, 11008, 12288, 14336, 16384, 22016, 28672, 32768]
 GRID_K = [2048, 4096, 5120, 8192, 11008, 14336, 28672]
 GRID_N_SMALL = [1, 4, 8, 12, 16]
-GRID_N_LARGE = [24, 32, 48, 64, 96, 128, 256, 512]
+GRID_N_LARGE = [24, 32, 48, 64, 96, 128, 256, 512, 1024, 2048]
 MAX_WEIGHTS = 28672 * 8192   # skip matrices beyond the largest layer of a 70B model
 
 
@@ -54,7 +54,7 @@ def candidates(OC, IC, BS):
     if BS <= 16:
         cfgs = STREAM_SMALL
     else:
-        cfgs = [c for c in TILE if c[1] * 16 < 2 * BS + 16 or c[1] == 2]
+        cfgs = [c for c in TILE if (c[1] * 16 < 2 * BS + 16 or c[1] == 2) and (BS <= 512 or c[1] >= 4)]
         if BS <= 32:
             cfgs = cfgs + STREAM_WIDE
     units = (IC + 255) // 256
@@ -64,7 +64,7 @@ def candidates(OC, IC, BS):
         for sk in SPLITS:
             if sk > units or (cfg[0] == 0 and sk > 1 and OC > 4096):   # the stream kernel splits K inside the workgroup already
                 continue
-            if sk > 1 and sk * 8 * BS > IC * 0.75:   # the FP32 partial sums would outweigh the weights themselves
+            if sk > 1 and (sk * 8 * BS > IC * 0.75 or BS > 512):   # the FP32 partial sums would outweigh the weights themselves
                 continue
             yield cfg, sk
 
