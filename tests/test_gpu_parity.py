@@ -302,6 +302,30 @@ def test_command_line_harness(E, M):
     assert res["splitK"] == 2 and res["max_rel_err_vs_fp32"] <= 1e-2
 
 
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_random_shapes_through_the_automatic_launch_choice(E, M):
+    """Forty seeded random problems per format -- rows in multiples of 256, columns in multiples of 64 (most of them not
+    multiples of 256, so the padded K block is exercised), batches from 1 to 300, the engine's own split or an arbitrary one --
+    through fp6mi_linear_native, whose launch shape comes from the measured table or the rules depending on the problem."""
+    rng = np.random.default_rng(2024 + E)
+    L = _lib.lib()
+    shape = (ctypes.c_int * 5)()
+    seen = set()
+    for case in range(40):
+        OC = 256 * int(rng.integers(1, 9))
+        IC = 64 * int(rng.integers(1, 49))
+        N = int(rng.choice([1, 2, 3, 5, 8, 9, 13, 16, 17, 24, 31, 33, 48, 64, 65, 100, 128, 130, 200, 300]))
+        splitK = fp6.heuristic_splitk_mi355x(OC, N, IC) if case % 3 else int(rng.integers(1, 7))
+        print("case random", E, M, OC, IC, N, splitK, flush=True)
+        raw, sc, x = synth.uniform_problem(7000 + case, OC, IC, N, E, M)
+        native, scd, xd = upload(raw, sc, x, E, M)
+        y = gemm_capi(E, M, native, scd, xd, OC, splitK)
+        check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "random %d: %dx%d N=%d splitK=%d" % (case, OC, IC, N, splitK))
+        assert L.fp6mi_query_launch(E, M, OC, N, IC, splitK, shape) == 0
+        seen.add(tuple(shape))
+    assert len(seen) >= 5   # the cases really spread over several kernel shapes
+
+
 # ------------------------------------------------------------------------------------------------ device-side quantizer
 def _awkward_weights(seed, OC, IC, dtype):
     """Gaussian weights with the cases a quantizer gets wrong: an all-zero row, a row of tiny values whose scale rounds to
