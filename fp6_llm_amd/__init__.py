@@ -10,17 +10,28 @@ fp6_llm/csrc/pybind.cpp:6-16):
 plus what the gfx950 engine adds: the native weight layout (``weight_prepacking_native_cpu``, ``to_native``,
 ``linear_forward_native``), a device-side dequantizer and a split-K heuristic derived for 256 compute units.
 
-Everything is computed by ``libfp6mi.so`` (C ABI in include/fp6mi.h) through ctypes; torch only owns memory and
-streams.  Where the reference aborts the process (assert / exit) these functions raise ``ValueError`` /
+Everything is computed by ``libfp6mi.so`` (C ABI in include/fp6mi.h).  The per-call GEMM path goes through a small torch
+C++ extension over that ABI (``_fp6mi_torch``, csrc/torch_binding.cpp) when it is built, else through ctypes -- the same
+library and kernels either way (``FP6MI_NO_TORCH_EXT=1`` forces ctypes); everything else uses ctypes.  Torch only owns
+memory and streams.  Where the reference aborts the process (assert / exit) these functions raise ``ValueError`` /
 ``RuntimeError`` instead.
 """
 import math
+import os
 import weakref
 
 import torch
 
 from . import _lib
 from ._lib import Fp6miError  # noqa: F401
+
+_lib.lib()   # fail at import, loudly, if the native library is missing; also makes libfp6mi.so resident for the extension
+_ext = None
+if not os.environ.get("FP6MI_NO_TORCH_EXT"):
+    try:
+        from . import _fp6mi_torch as _ext
+    except ImportError:   # not built (it needs torch's headers at build time): the ctypes path below does the same job
+        _ext = None
 
 __all__ = [
     "linear_forward_cuda", "weight_prepacking_cpu", "weight_dequant_cpu",
@@ -199,6 +210,8 @@ _native_cache = {}  # id(tensor) -> (weakref, version, data_ptr, E, M, native te
 def clear_caches():
     _workspaces.clear()
     _native_cache.clear()
+    if _ext is not None:
+        _ext.clear_workspaces()
 
 
 def _workspace(device, stream, nbytes):
@@ -215,6 +228,8 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the curre
 
 def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, splitK=1, out=None, workspace=None):
     """out[B, OC] = in_feats[B, IC] @ dequant(W)^T with W in the native layout.  Enqueued on the current stream."""
+    if _ext is not None:
+        return _ext.linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, int(splitK), out, workspace)
     _bits(EXPONENT, MANTISSA)
     if in_feats.dtype != torch.float16 or in_feats.dim() != 2:
         raise ValueError("in_feats must be a 2-D float16 tensor [B, IC]")

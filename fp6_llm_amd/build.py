@@ -34,10 +34,38 @@ def _compile(sources, output, verbose):
     return output
 
 
+def build_torch_extension(verbose=False):
+    """Compiles csrc/torch_binding.cpp (a host-only translation unit: g++, torch's headers, the C ABI) into
+    _fp6mi_torch.so next to libfp6mi.so, which must exist."""
+    import sysconfig
+
+    from torch.utils import cpp_extension as ce
+    import torch
+
+    out = os.path.join(HERE, "_fp6mi_torch.so")
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1", "-DTORCH_EXTENSION_NAME=_fp6mi_torch",
+           "-DTORCH_API_INCLUDE_EXTENSION_H", "-D_GLIBCXX_USE_CXX11_ABI=%d" % int(torch.compiled_with_cxx11_abi())]
+    cmd += ["-I" + p for p in ce.include_paths()] + ["-I" + sysconfig.get_paths()["include"], "-I/opt/rocm/include", "-I" + os.path.join(ROOT, "include")]
+    cmd += [os.path.join(HERE, "csrc", "torch_binding.cpp")]
+    libdirs = ce.library_paths()
+    cmd += ["-L" + p for p in libdirs] + ["-ltorch", "-ltorch_cpu", "-ltorch_python", "-lc10", "-lc10_hip", "-L" + HERE, "-lfp6mi", "-Wl,-rpath,$ORIGIN"]
+    cmd += ["-Wl,-rpath," + p for p in libdirs] + ["-o", out + ".tmp"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if verbose or res.returncode != 0:
+        sys.stderr.write(res.stdout + res.stderr)
+    if res.returncode != 0:
+        raise RuntimeError("g++ failed building _fp6mi_torch.so")
+    os.replace(out + ".tmp", out)
+    return out
+
+
 def build(verbose=False):
-    """Compiles every HIP/C++ source for gfx950 into libfp6mi.so and libfp6mi_probe.so (always recompiles)."""
+    """Compiles every HIP/C++ source for gfx950 into libfp6mi.so and libfp6mi_probe.so, then the torch extension over the C
+    ABI (always recompiles)."""
     _compile(PROBE_SOURCES, PROBE_OUTPUT, verbose)
-    return _compile(SOURCES, OUTPUT, verbose)
+    lib = _compile(SOURCES, OUTPUT, verbose)
+    build_torch_extension(verbose)
+    return lib
 
 
 if __name__ == "__main__":

@@ -233,6 +233,27 @@ def test_c_abi_drop_in_on_reference_layout(E, M):
     assert L.fp6mi_twin_clear() == 0
 
 
+def test_torch_extension_and_ctypes_binding_agree(monkeypatch):
+    """The per-call path exists twice over the same C ABI: the torch C++ extension (used when built) and ctypes."""
+    assert fp6._ext is not None, "fp6_llm_amd/_fp6mi_torch.so is built by python -m fp6_llm_amd.build"
+    E, M, OC, IC = 3, 2, 512, 1280
+    for N, splitK in ((5, 1), (40, 3)):
+        raw, sc, x = synth.uniform_problem(900 + N, OC, IC, N, E, M)
+        native, scd, xd = upload(raw, sc, x, E, M)
+        y_ext = fp6.linear_forward_native(E, M, xd, native, scd, OC, splitK)
+        with pytest.raises(ValueError):
+            fp6.linear_forward_native(E, M, xd.float(), native, scd, OC, splitK)
+        with pytest.raises(ValueError):
+            fp6.linear_forward_native(E, M, xd, native[:-1], scd, OC, splitK)
+        monkeypatch.setattr(fp6, "_ext", None)
+        y_ct = fp6.linear_forward_native(E, M, xd, native, scd, OC, splitK)
+        with pytest.raises(ValueError):
+            fp6.linear_forward_native(E, M, xd.float(), native, scd, OC, splitK)
+        monkeypatch.undo()
+        assert torch.equal(y_ext, y_ct)
+        check_close(y_ext.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "extension path N=%d" % N)
+
+
 def test_cpp_api_driver():
     """The reference-named C++ API (fp6_llm_amd/csrc/fp6_linear.h) through the command-line driver, in the order the
     reference's C++ test uses it: dequantize, prepack in place, upload, GEMM."""
