@@ -15,7 +15,7 @@ Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth fi
 on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
 launch stream; `cpu_baseline` times the reference's CPU path (dequantize, then a torch CPU matmul) on this host;
 `detail.read_floor_us` is the time of a kernel that only reads the same weight buffers the same way (no arithmetic).
---sweep additionally runs every benchmark configuration and writes gpurun_out/bench_sweep.jsonl.
+--sweep additionally runs every benchmark configuration and writes one JSON line per configuration to --sweep-out.
 """
 import argparse
 import json
@@ -363,7 +363,8 @@ def main():
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
-    ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration (writes gpurun_out/bench_sweep.jsonl)")
+    ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration")
+    ap.add_argument("--sweep-out", default="bench_sweep.jsonl", help="where --sweep writes its JSON lines")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the legs that run outside this process's GPU stream: the CPU path and the system-BLAS FP16 baseline (a child process)")
     ap.add_argument("--warm", action="store_true", help="also time the workload with the same weight buffer every step (cache-resident weights)")
@@ -403,8 +404,8 @@ def main():
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(E, M, OC, IC, BS)
     if args.sweep:
-        os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-        with open(os.path.join(ROOT, "gpurun_out", "bench_sweep.jsonl"), "w") as f:
+        os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
+        with open(args.sweep_out, "w") as f:
             for name in WORKLOADS:
                 big = WORKLOADS[name][2] * WORKLOADS[name][3] > 64e6
                 r, _ = run_workload(name, 100 if big else 300, 10, device)
