@@ -25,10 +25,13 @@ import torch
 from . import _lib
 from ._lib import Fp6miError  # noqa: F401
 
-_lib.lib()   # fail at import, loudly, if the native library is missing; also makes libfp6mi.so resident for the extension
+# The native library is loaded on first use (every entry point raises ImportError while it is missing: there is no other
+# path), so that `python -m fp6_llm_amd.build` can import this package before anything is built.  The torch extension links
+# against it and is only tried once it is there.
 _ext = None
-if not os.environ.get("FP6MI_NO_TORCH_EXT"):
+if os.path.exists(_lib.LIB_PATH) and not os.environ.get("FP6MI_NO_TORCH_EXT"):
     try:
+        _lib.lib()
         from . import _fp6mi_torch as _ext
     except ImportError:   # not built (it needs torch's headers at build time): the ctypes path below does the same job
         _ext = None
