@@ -14,6 +14,7 @@
 
 #include <mutex>
 #include <unordered_map>
+#include <vector>
 
 #include "fp6mi_internal.h"
 
@@ -782,32 +783,48 @@ inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (
 
 // Nearest measured problem: the batch is rounded UP to a measured batch of the same kernel family (a shape's cost steps at
 // column-tile boundaries), M and K go to the nearest measured value in ratio, at most a factor 1.5 away.
+struct TuneGroup { int xb; size_t n, begin, end; }; // entries [begin, end) of kTune share format and batch (the table is sorted by them)
+
+const std::vector<TuneGroup> &tune_groups()
+{
+    static const std::vector<TuneGroup> groups = [] {
+        std::vector<TuneGroup> g;
+        const size_t           count = sizeof(kTune) / sizeof(kTune[0]);
+        for (size_t i = 1; i < count; i++) {
+            if (g.empty() || g.back().xb != kTune[i].xb || g.back().n != kTune[i].n) g.push_back(TuneGroup{ kTune[i].xb, kTune[i].n, i, i });
+            g.back().end = i + 1;
+        }
+        return g;
+    }();
+    return groups;
+}
+
 const TuneEntry *tune_lookup(int xbits, size_t M, size_t N, size_t K)
 {
+    // a serving loop asks for the same few layer shapes at whatever batch size the scheduler formed: remember answers
     struct Memo { int xb; size_t M, N, K; const TuneEntry *e; };
-    static thread_local Memo memo[8];
-    static thread_local unsigned next = 0;
-    for (const Memo &m : memo)
-        if (m.xb == xbits && m.M == M && m.N == N && m.K == K) return m.e;
-    const size_t count = sizeof(kTune) / sizeof(kTune[0]);
-    size_t       n_target = 0, n_max = 0;
-    for (size_t i = 1; i < count; i++) {
-        const TuneEntry &e = kTune[i];
-        if (e.xb != xbits || (e.n <= 16) != (N <= 16)) continue;
-        if (e.n >= N && (n_target == 0 || e.n < n_target)) n_target = e.n;
-        if (e.n > n_max) n_max = e.n;
+    static thread_local Memo memo[256];
+    Memo &slot = memo[(M * 0x9E3779B97F4A7C15ull + N * 0xC2B2AE3D27D4EB4Full + K * 0x165667B19E3779F9ull + (size_t)xbits) >> 56];
+    if (slot.xb == xbits && slot.M == M && slot.N == N && slot.K == K) return slot.e;
+    const TuneGroup *group = nullptr, *widest = nullptr;
+    for (const TuneGroup &g : tune_groups()) {
+        if (g.xb != xbits || (g.n <= 16) != (N <= 16)) continue;
+        if (g.n >= N && (!group || g.n < group->n)) group = &g;
+        if (!widest || g.n > widest->n) widest = &g;
     }
-    if (n_target == 0) n_target = n_max; // batches beyond the largest measured one behave like it, only more column blocks
+    if (!group) group = widest; // batches beyond the largest measured one behave like it, only with more column blocks
     const TuneEntry *best = nullptr;
     float            best_d = 0.f;
-    for (size_t i = 1; n_target && i < count; i++) {
-        const TuneEntry &e = kTune[i];
-        if (e.xb != xbits || e.n != n_target) continue;
-        float dm = std::fabs(std::log2((float)M / (256.f * e.m256))), dk = std::fabs(std::log2((float)K / (64.f * e.k64)));
-        if (dm > 0.585f || dk > 0.585f) continue;
-        if (!best || dm + dk < best_d) { best = &e; best_d = dm + dk; }
+    if (group) {
+        const float lm = std::log2((float)M / 256.f), lk = std::log2((float)K / 64.f);
+        for (size_t i = group->begin; i < group->end; i++) {
+            const TuneEntry &e = kTune[i];
+            float dm = std::fabs(lm - std::log2((float)e.m256)), dk = std::fabs(lk - std::log2((float)e.k64));
+            if (dm > 0.585f || dk > 0.585f) continue;
+            if (!best || dm + dk < best_d) { best = &e; best_d = dm + dk; }
+        }
     }
-    memo[next++ % 8] = Memo{ xbits, M, N, K, best };
+    slot = Memo{ xbits, M, N, K, best };
     return best;
 }
 
