@@ -335,3 +335,20 @@ def test_bench_refuses_more_than_one_gpu_and_lists_the_benchmark_configurations(
     # 70B shapes at 32, and 8192^2 at ten batch sizes in both formats
     assert len(bench.WORKLOADS) == 3 + 4 + 3 + 20
     assert bench.weight_bytes(3, 2, 4096, 4096) == 12582912 and bench.algorithmic_bytes(3, 2, 4096, 4096, 8) == 12722176
+
+
+def test_tuner_candidates_and_table_emission(tmp_path, monkeypatch):
+    from fp6_llm_amd import tune
+    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE)
+    for (OC, IC, BS) in [(256, 64, 1), (4096, 4096, 8), (4096, 4096, 17), (11008, 4096, 64), (768, 2048, 512), (8192, 8192, 2048)]:
+        cands = list(tune.candidates(OC, IC, BS))
+        assert cands, (OC, IC, BS)
+        for cfg, sk in cands:
+            assert cfg in compiled and OC % tune.tile_rows(cfg) == 0 and 1 <= sk <= (IC + 255) // 256
+            assert (cfg[0] == 0) == (BS <= 16 or cfg in tune.STREAM_WIDE)
+    src = tmp_path / "t.jsonl"
+    src.write_text(json.dumps({"E": 3, "M": 2, "OC": 512, "IC": 1024, "BS": 8, "best": {"1": [[0, 1, 1, 1, 8], 3.21], "4": [[0, 1, 2, 1, 4], 4.0]}}) + "\n")
+    monkeypatch.setattr(tune, "INC_PATH", str(tmp_path / "out.inc"))
+    tune.main(["emit", str(src)])
+    lines = [l for l in (tmp_path / "out.inc").read_text().splitlines() if l.startswith("{")]
+    assert lines == ["{6,2,16,8,{{0,1,1,1,8,160},{255,0,0,0,0,0},{0,1,2,1,4,200},{255,0,0,0,0,0}}},"]
