@@ -48,6 +48,10 @@ WORKLOADS = {
 for _bs in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512):
     WORKLOADS["fp6_8192x8192_bs%d" % _bs] = (3, 2, 8192, 8192, _bs)
     WORKLOADS["fp5_8192x8192_bs%d" % _bs] = (2, 2, 8192, 8192, _bs)
+for _bs in (1, 8, 32, 128):   # the two formats beyond the reference's: same shapes, for the sweep
+    WORKLOADS["fp6e2m3_8192x8192_bs%d" % _bs] = (2, 3, 8192, 8192, _bs)
+    WORKLOADS["fp4_8192x8192_bs%d" % _bs] = (2, 1, 8192, 8192, _bs)
+WORKLOADS["fp4_4096x4096_bs8"] = (2, 1, 4096, 4096, 8)
 HEADLINE = "fp6_4096x4096_bs8"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
@@ -395,8 +399,8 @@ def main():
         "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["us_per_gemm"] / 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "%s: FP%d_e%dm2 weights [%d,%d] x fp16 activations [%d,%d], weights rotating through %d distinct HBM buffers, splitK=%d"
-                               % (args.workload, 1 + E + M, E, OC, IC, BS, IC, res["weight_buffers"], res["splitK"])},
+        "config": {"workload": "%s: FP%d_e%dm%d weights [%d,%d] x fp16 activations [%d,%d], weights rotating through %d distinct HBM buffers, splitK=%d"
+                               % (args.workload, 1 + E + M, E, M, OC, IC, BS, IC, res["weight_buffers"], res["splitK"])},
         "roofline": {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
                      "bytes_per_launch": res["weight_bytes"], "kernel_us": res["us_per_gemm"]},
         "detail": res,

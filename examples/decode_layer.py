@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """The linear layers of one transformer decoder layer at decode batch sizes, FPx weights against FP16 weights.
 
-    python examples/decode_layer.py [--model 7b|70b] [--format 6|5] [--batch 1,8,32]
+    python examples/decode_layer.py [--model 7b|70b] [--format 6|5|4] [--batch 1,8,32]
 
 Builds the four GEMMs of a LLaMA-shaped layer as `FPxLinear` modules -- Q, K and V fused into one launch and gate and up
 into another with `FPxLinear.fused` -- quantizes random weights on the GPU, captures one pass over the four layers into a
@@ -52,12 +52,12 @@ def timed_graph(fn, copies, reps=20):
 def main():
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     ap.add_argument("--model", default="7b", choices=sorted(SHAPES))
-    ap.add_argument("--format", type=int, default=6, choices=(5, 6))
+    ap.add_argument("--format", type=int, default=6, choices=(4, 5, 6), help="6 = FP6_e3m2, 5 = FP5_e2m2, 4 = FP4_e2m1")
     ap.add_argument("--batch", default="1,8,32")
     args = ap.parse_args()
     dims = SHAPES[args.model]
     H, KV, F = dims["hidden"], dims["kv"], dims["mlp"]
-    E, M = (3, 2) if args.format == 6 else (2, 2)
+    E, M = {6: (3, 2), 5: (2, 2), 4: (2, 1)}[args.format]
     dev = torch.device("cuda:0")
     layer_bytes_fp16 = 2 * (H * (H + 2 * KV) + H * H + 2 * F * H + H * F)
     copies = max(2, min(16, (1 << 30) // layer_bytes_fp16 + 1))   # > 256 MB of distinct weights per pass over the copies
@@ -72,8 +72,8 @@ def main():
         return fpx, f16
 
     layers = [make(c) for c in range(copies)]
-    print("LLaMA-%s-shaped layer, FP%d_e%dm2 vs FP16, %d weight copies rotating (%.0f MB of FP16 weights per layer)"
-          % (args.model, 1 + E + M, E, copies, layer_bytes_fp16 / 1e6))
+    print("LLaMA-%s-shaped layer, FP%d_e%dm%d vs FP16, %d weight copies rotating (%.0f MB of FP16 weights per layer)"
+          % (args.model, 1 + E + M, E, M, copies, layer_bytes_fp16 / 1e6))
     for B in [int(b) for b in args.batch.split(",")]:
         x_h = torch.randn(B, H, device=dev, dtype=torch.float16)
         x_f = torch.randn(B, F, device=dev, dtype=torch.float16)

@@ -72,9 +72,15 @@ def heuristic_splitk_mi355x(M, N, K, num_cus=MI355X_CUS):
 # ----------------------------------------------------------------------------------------------------------------
 # helpers
 # ----------------------------------------------------------------------------------------------------------------
+# FP6_e3m2 and FP5_e2m2 are the reference's formats (fp6_llm/csrc/fp6_linear.cu:133-138); FP6_e2m3 and FP4_e2m1 run through
+# the same entry points here.
+FORMATS = ((3, 2), (2, 2), (2, 3), (2, 1))
+_BLOCK_BYTES = {6: 3072, 5: 2560, 4: 2048}   # bytes of a 16-row x 256-column block of the native layout, by bit width
+
+
 def _bits(E, M):
-    if (E, M) not in ((3, 2), (2, 2)):
-        raise ValueError("unsupported format: EXPONENT=%d, MANTISSA=%d (only e3m2 and e2m2)" % (E, M))
+    if (E, M) not in FORMATS:
+        raise ValueError("unsupported format: EXPONENT=%d, MANTISSA=%d (only e3m2, e2m2, e2m3 and e2m1)" % (E, M))
     return 1 + E + M
 
 
@@ -170,7 +176,7 @@ def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC
     _bits(EXPONENT, MANTISSA)
     if native_weight.device.type != "cuda" or fp16_scale.device != native_weight.device:
         raise ValueError("native_weight and fp16_scale must be on the same GPU")
-    if native_weight.numel() * native_weight.element_size() != native_bytes(EXPONENT, MANTISSA, OC, IC):
+    if native_weight.numel() * native_weight.element_size() != (OC // 16) * ((IC + 255) // 256) * _BLOCK_BYTES[1 + EXPONENT + MANTISSA]:
         raise ValueError("native_weight has the wrong size for OC=%d IC=%d" % (OC, IC))
     out = torch.empty((OC, IC), dtype=torch.float16, device=native_weight.device)
     with torch.cuda.device(native_weight.device):
@@ -248,7 +254,7 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
         raise ValueError("need OC %% 256 == 0, IC %% 64 == 0, B >= 1 (got OC=%d IC=%d B=%d)" % (OC, IC, B))
     # same value as fp6mi_native_bytes, computed here: this function is on the per-token path and a 5 us kernel deserves a
     # wrapper that costs less than it does
-    if native_weight.numel() * native_weight.element_size() != (OC // 16) * ((IC + 255) // 256) * (3072 if EXPONENT == 3 else 2560):
+    if native_weight.numel() * native_weight.element_size() != (OC // 16) * ((IC + 255) // 256) * _BLOCK_BYTES[1 + EXPONENT + MANTISSA]:
         raise ValueError("native_weight has the wrong size for OC=%d IC=%d" % (OC, IC))
     splitK = int(splitK)
     if splitK < 1:

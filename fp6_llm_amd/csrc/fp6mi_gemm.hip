@@ -8,11 +8,13 @@
 // to VGPRs with 128-bit non-temporal loads, FP6 codes are converted by the CDNA4 instruction
 // v_cvt_scalef32_pk32_f16_bf6 (BF6 = e3m2, bias 3, no inf/nan: the very format of the reference), FP5 codes by the same
 // instruction after a zero bit is slipped in above their exponent (an e2m2 code read as e3m2 is a quarter of its value),
-// and v_mfma_f32_16x16x32_f16 accumulates in FP32.  The per-row scale (and the factor 4 of FP5) is applied once to the
-// FP32 sums instead of to every weight.
+// FP6_e2m3 codes by v_cvt_scalef32_pk32_f16_fp6 and FP4_e2m1 codes by that instruction after two zero bits are appended
+// to their mantissa, and v_mfma_f32_16x16x32_f16 accumulates in FP32.  The per-row scale (and the factor 4 of FP5) is
+// applied once to the FP32 sums instead of to every weight.
 #include <hip/hip_runtime.h>
 
 #include <mutex>
+#include <type_traits>
 #include <unordered_map>
 #include <vector>
 
@@ -30,38 +32,39 @@ typedef uint32_t v6u __attribute__((ext_vector_type(6)));
 
 constexpr int kWave = 64;
 
-template <int XB> struct Fmt;
-template <> struct Fmt<6> { static constexpr int block_bytes = 3072; static constexpr float post_scale = 1.0f; };
-template <> struct Fmt<5> { static constexpr int block_bytes = 2560; static constexpr float post_scale = 4.0f; };
+// Formats are named by the tag FM = 10*E + M.  `hw_e3m2` says which conversion instruction reads the 6-bit fields that the
+// native layout holds (BF6 = e3m2 or FP6 = e2m3); post_scale is the factor the epilogue owes the sums.
+template <int FM> struct Fmt;
+template <> struct Fmt<32> { static constexpr int bits = 6, man = 2, bias = 3, block_bytes = 3072; static constexpr bool hw_e3m2 = true;
+                             static constexpr float post_scale = 1.0f; static constexpr double max_value = 28.0; };
+template <> struct Fmt<22> { static constexpr int bits = 5, man = 2, bias = 1, block_bytes = 2560; static constexpr bool hw_e3m2 = true;
+                             static constexpr float post_scale = 4.0f; static constexpr double max_value = 7.0; };
+template <> struct Fmt<23> { static constexpr int bits = 6, man = 3, bias = 1, block_bytes = 3072; static constexpr bool hw_e3m2 = false;
+                             static constexpr float post_scale = 1.0f; static constexpr double max_value = 7.5; };
+template <> struct Fmt<21> { static constexpr int bits = 4, man = 1, bias = 1, block_bytes = 2048; static constexpr bool hw_e3m2 = false;
+                             static constexpr float post_scale = 1.0f; static constexpr double max_value = 6.0; };
 
 // The weights of one lane for one 16x256 block, as loaded from memory.
-template <int XB> struct WFrag;
-template <> struct WFrag<6> { v4u a, b, c; };
-template <> struct WFrag<5> { v4u a, b; v2u s; };
+template <int FM> struct WFrag;
+template <> struct WFrag<32> { v4u a, b, c; };
+template <> struct WFrag<23> { v4u a, b, c; };
+template <> struct WFrag<22> { v4u a, b; v2u s; };
+template <> struct WFrag<21> { v4u a, b; };
 
-template <int XB> __device__ __forceinline__ WFrag<XB> load_wfrag(const uint8_t *block, int lane);
-template <> __device__ __forceinline__ WFrag<6> load_wfrag<6>(const uint8_t *block, int lane)
+template <int FM> __device__ __forceinline__ WFrag<FM> load_wfrag(const uint8_t *block, int lane)
 {
     const v4u *p = reinterpret_cast<const v4u *>(block) + lane;
-    WFrag<6>   f;
+    WFrag<FM>  f;
     f.a = __builtin_nontemporal_load(p);
     f.b = __builtin_nontemporal_load(p + 64);
-    f.c = __builtin_nontemporal_load(p + 128);
-    return f;
-}
-template <> __device__ __forceinline__ WFrag<5> load_wfrag<5>(const uint8_t *block, int lane)
-{
-    const v4u *p = reinterpret_cast<const v4u *>(block) + lane;
-    WFrag<5>   f;
-    f.a = __builtin_nontemporal_load(p);
-    f.b = __builtin_nontemporal_load(p + 64);
-    f.s = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(block + 2048) + lane);
+    if constexpr (Fmt<FM>::bits == 6) f.c = __builtin_nontemporal_load(p + 128);
+    if constexpr (Fmt<FM>::bits == 5) f.s = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(block + 2048) + lane);
     return f;
 }
 
 // A operands (8 halfs = k 8q..8q+7 of this lane's row) of the eight MFMA steps of a block.
-// FP6: exact values.  FP5: a quarter of the values (exact; the epilogue multiplies the sums by 4).
-template <int XB> struct AOps { v8h s[8]; };
+// FP5: a quarter of the values (exact; the epilogue multiplies the sums by 4).  The other formats: exact values.
+template <int FM> struct AOps { v8h s[8]; };
 
 __device__ __forceinline__ v8h slice8(const v32h &v, int i)
 {
@@ -70,19 +73,6 @@ __device__ __forceinline__ v8h slice8(const v32h &v, int i)
     case 1: return __builtin_shufflevector(v, v, 8, 9, 10, 11, 12, 13, 14, 15);
     case 2: return __builtin_shufflevector(v, v, 16, 17, 18, 19, 20, 21, 22, 23);
     default: return __builtin_shufflevector(v, v, 24, 25, 26, 27, 28, 29, 30, 31);
-    }
-}
-
-__device__ __forceinline__ void convert(const WFrag<6> &f, AOps<6> &o)
-{
-    v6u  lo = { f.a[0], f.a[1], f.a[2], f.a[3], f.b[0], f.b[1] };
-    v6u  hi = { f.b[2], f.b[3], f.c[0], f.c[1], f.c[2], f.c[3] };
-    v32h h0 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(lo, 1.0f);
-    v32h h1 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(hi, 1.0f);
-#pragma unroll
-    for (int i = 0; i < 4; i++) {
-        o.s[i]     = slice8(h0, i);
-        o.s[4 + i] = slice8(h1, i);
     }
 }
 
@@ -95,10 +85,37 @@ __device__ __forceinline__ v6u fp5_expand(uint32_t s0, uint32_t s1, uint32_t s2,
     return (v6u){ s0 & ~A, s1 & ~B, s2 & ~C, s3 & ~A, s4 & ~B, (hi << 1) | lo };
 }
 
-__device__ __forceinline__ void convert(const WFrag<5> &f, AOps<5> &o)
+// FP4: 32 codes are stored in four dwords; the fifth and sixth dword of the 6-bit string sit in the fixed-zero bit pairs (the
+// two bits appended below every mantissa) of the other four, at their own bit positions (layout: fp6mi_host.cpp).
+__device__ __forceinline__ v6u fp4_expand(v4u s)
 {
-    v32h h0 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(fp5_expand(f.a[0], f.a[1], f.a[2], f.a[3], f.s[0]), 1.0f);
-    v32h h1 = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(fp5_expand(f.b[0], f.b[1], f.b[2], f.b[3], f.s[1]), 1.0f);
+    constexpr uint32_t P = 0xC30C30C3u, Q = 0x30C30C30u, R = 0x0C30C30Cu;
+    return (v6u){ s[0] & ~P, s[1] & ~Q, s[2] & ~R, s[3] & ~P, (s[0] & P) | (s[2] & R), (s[1] & Q) | (s[3] & P) };
+}
+
+// The 192-bit string of 6-bit fields of MFMA steps 4h..4h+3 (half of a K block) of one lane, and its conversion.
+template <int FM> __device__ __forceinline__ v6u field_string(const WFrag<FM> &f, int h)
+{
+    if constexpr (Fmt<FM>::bits == 6)
+        return h == 0 ? (v6u){ f.a[0], f.a[1], f.a[2], f.a[3], f.b[0], f.b[1] } : (v6u){ f.b[2], f.b[3], f.c[0], f.c[1], f.c[2], f.c[3] };
+    else if constexpr (Fmt<FM>::bits == 5)
+        return h == 0 ? fp5_expand(f.a[0], f.a[1], f.a[2], f.a[3], f.s[0]) : fp5_expand(f.b[0], f.b[1], f.b[2], f.b[3], f.s[1]);
+    else
+        return fp4_expand(h == 0 ? f.a : f.b);
+}
+
+template <int FM> __device__ __forceinline__ v32h fields_to_halfs(v6u src)
+{
+    if constexpr (Fmt<FM>::hw_e3m2)
+        return __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
+    else
+        return __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(src, 1.0f);
+}
+
+template <int FM> __device__ __forceinline__ void convert(const WFrag<FM> &f, AOps<FM> &o)
+{
+    v32h h0 = fields_to_halfs<FM>(field_string<FM>(f, 0));
+    v32h h1 = fields_to_halfs<FM>(field_string<FM>(f, 1));
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         o.s[i]     = slice8(h0, i);
@@ -131,17 +148,17 @@ template <int NT> __device__ __forceinline__ void load_x_paired(v8h (&x)[8][NT],
     }
 }
 
-template <int XB, int NT, int RT> struct Stage {
-    WFrag<XB> w[RT];
+template <int FM, int NT, int RT> struct Stage {
+    WFrag<FM> w[RT];
     v8h       x[8][NT];
 };
 
-template <int XB, int NT, int RT>
-__device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
+template <int FM, int NT, int RT>
+__device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
                                            const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack, const half_t *xrow_packed)
 {
 #pragma unroll
-    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
+    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
     // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
@@ -165,12 +182,12 @@ __device__ __forceinline__ void load_stage(Stage<XB, NT, RT> &st, const uint8_t 
     __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
 }
 
-template <int XB, int NT, int RT>
-__device__ __forceinline__ void consume_stage(const Stage<XB, NT, RT> &st, v4f (&acc)[RT][NT])
+template <int FM, int NT, int RT>
+__device__ __forceinline__ void consume_stage(const Stage<FM, NT, RT> &st, v4f (&acc)[RT][NT])
 {
 #pragma unroll
     for (int r = 0; r < RT; r++) {
-        AOps<XB> a;
+        AOps<FM> a;
         convert(st.w[r], a);
 #pragma unroll
         for (int s = 0; s < 8; s++)
@@ -179,7 +196,7 @@ __device__ __forceinline__ void consume_stage(const Stage<XB, NT, RT> &st, v4f (
     }
 }
 
-template <int XB, int NT, int RT, int WAVES>
+template <int FM, int NT, int RT, int WAVES>
 __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
                                                             const half_t *__restrict__ X, half_t *__restrict__ C,
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
@@ -195,7 +212,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     const uint32_t u0 = split * avg + (split < extra ? split : extra);
     const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
 
-    const size_t   tile_stride = (size_t)units * Fmt<XB>::block_bytes;
+    const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
 
     v4f acc[RT][NT];
@@ -230,9 +247,9 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     // One K block at a time and no register double-buffering: the other wavefronts of the workgroup keep the memory system
     // busy while this one converts, and a second stage in registers measured slower at every size.
     for (uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES); u < u1; u += WAVES) {
-        Stage<XB, NT, RT> cur;
-        load_stage<XB, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
-        consume_stage<XB, NT, RT>(cur, acc);
+        Stage<FM, NT, RT> cur;
+        load_stage<FM, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
+        consume_stage<FM, NT, RT>(cur, acc);
     }
 
     // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
@@ -254,7 +271,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         for (int w = 0; w < WAVES; w++) sum += red[w][rt][idx];
         uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
         if (ng < N) {
-            float v = sum * ((float)my_scale[j] * Fmt<XB>::post_scale);
+            float v = sum * ((float)my_scale[j] * Fmt<FM>::post_scale);
             if (splitK == 1)
                 C[(size_t)ng * M + mg] = (half_t)v;
             else
@@ -264,17 +281,9 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 }
 
 // A operands of MFMA steps 4h..4h+3 (half of a K block) of one lane.
-__device__ __forceinline__ void convert_half(const WFrag<6> &f, int h, v8h (&o)[4])
+template <int FM> __device__ __forceinline__ void convert_half(const WFrag<FM> &f, int h, v8h (&o)[4])
 {
-    v6u src = h == 0 ? (v6u){ f.a[0], f.a[1], f.a[2], f.a[3], f.b[0], f.b[1] } : (v6u){ f.b[2], f.b[3], f.c[0], f.c[1], f.c[2], f.c[3] };
-    v32h v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
-#pragma unroll
-    for (int i = 0; i < 4; i++) o[i] = slice8(v, i);
-}
-__device__ __forceinline__ void convert_half(const WFrag<5> &f, int h, v8h (&o)[4])
-{
-    v6u  src = h == 0 ? fp5_expand(f.a[0], f.a[1], f.a[2], f.a[3], f.s[0]) : fp5_expand(f.b[0], f.b[1], f.b[2], f.b[3], f.s[1]);
-    v32h v = __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
+    v32h v = fields_to_halfs<FM>(field_string<FM>(f, h));
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = slice8(v, i);
 }
@@ -293,7 +302,7 @@ __device__ __forceinline__ void convert_half(const WFrag<5> &f, int h, v8h (&o)[
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kXsRowBytes = 544;
 
-template <int XB, int NT, int RT, int WR, int WK>
+template <int FM, int NT, int RT, int WR, int WK>
 __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
                                                            const half_t *__restrict__ X, half_t *__restrict__ C,
                                                            float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
@@ -319,7 +328,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     const uint32_t u0 = split * avg + (split < extra ? split : extra);
     const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
 
-    const size_t   tile_stride = (size_t)units * Fmt<XB>::block_bytes;
+    const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
 
     v4f acc[RT][NT];
@@ -328,7 +337,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
         for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
 
-    WFrag<XB> wcur[RT], wnxt[RT];
+    WFrag<FM> wcur[RT], wnxt[RT];
     v4u       xr[kPerThread];
 
     // row scales of this lane's outputs (rows 4q..4q+3 of each of its row tiles), fetched before the main loop so that no
@@ -338,11 +347,11 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
     for (int r = 0; r < RT; r++) sc4[r] = *reinterpret_cast<const v4h *>(scales + (R0 + r) * 16 + 4 * q);
 
-    auto load_w = [&](WFrag<XB>(&dst)[RT], uint32_t c0) {
+    auto load_w = [&](WFrag<FM>(&dst)[RT], uint32_t c0) {
         const uint32_t u = c0 + wk;
         if (u < u1) {
 #pragma unroll
-            for (int r = 0; r < RT; r++) dst[r] = load_wfrag<XB>(wgroup + r * tile_stride + (size_t)u * Fmt<XB>::block_bytes, lane);
+            for (int r = 0; r < RT; r++) dst[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
         }
     };
     // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
@@ -452,7 +461,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
                 if (ng < N) {
                     v4f v;
 #pragma unroll
-                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<XB>::post_scale);
+                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
                     if (splitK == 1) {
                         v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
                         *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
@@ -478,7 +487,7 @@ __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, con
 }
 
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
-template <int XB>
+template <int FM>
 __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, const uint8_t *__restrict__ W,
                                                      const half_t *__restrict__ scales, uint32_t M, uint32_t K, uint32_t units)
 {
@@ -487,16 +496,16 @@ __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, 
     if (blk >= (M / 16) * units) return;
     const uint32_t R = blk / units, U = blk % units;
     const int      m = lane & 15, q = lane >> 4;
-    WFrag<XB>      wf = load_wfrag<XB>(W + (size_t)blk * Fmt<XB>::block_bytes, lane);
-    AOps<XB>       a;
+    WFrag<FM>      wf = load_wfrag<FM>(W + (size_t)blk * Fmt<FM>::block_bytes, lane);
+    AOps<FM>       a;
     convert(wf, a);
-    const half_t sc = scales[R * 16 + m], post = (half_t)Fmt<XB>::post_scale;
+    const half_t sc = scales[R * 16 + m], post = (half_t)Fmt<FM>::post_scale;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
         uint32_t k = U * 256 + 32 * s + 8 * q;
         if (k < K) {
             v8h v = a.s[s];
-            if (XB == 5) v = v * post; // exact: a power of two, results are at most 7
+            if (Fmt<FM>::post_scale != 1.0f) v = v * post; // exact: a power of two, results are at most 7
             v = v * sc;                // one round-to-nearest-even, like fp16_rn(value * scale)
             *reinterpret_cast<v8h *>(out + (size_t)(R * 16 + m) * K + k) = v;
         }
@@ -504,10 +513,10 @@ __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, 
 }
 
 // Writes the 64 codes of one lane (c[8*s + j] = code of its row at column 32*s + 8*q + j of the K block) as the lane's
-// 12 (FP6) or 10 (FP5) dwords of a native block.
-template <int XB> __device__ __forceinline__ void store_native_lane(const uint8_t (&c)[64], uint8_t *dst, int lane)
+// 12 (6-bit formats), 10 (FP5) or 8 (FP4) dwords of a native block.
+template <int FM> __device__ __forceinline__ void store_native_lane(const uint8_t (&c)[64], uint8_t *dst, int lane)
 {
-    if (XB == 6) {
+    if (Fmt<FM>::bits == 6) {
         uint32_t d[12];
         for (int h = 0; h < 2; h++) {
             uint64_t accb = 0;
@@ -521,6 +530,20 @@ template <int XB> __device__ __forceinline__ void store_native_lane(const uint8_
         for (int i = 0; i < 3; i++) {
             v4u v = { d[4 * i], d[4 * i + 1], d[4 * i + 2], d[4 * i + 3] };
             reinterpret_cast<v4u *>(dst)[i * 64 + lane] = v;
+        }
+    } else if (Fmt<FM>::bits == 4) {
+        constexpr uint32_t P = 0xC30C30C3u, Q = 0x30C30C30u, R = 0x0C30C30Cu;
+        for (int h = 0; h < 2; h++) {
+            uint32_t D[6];
+            uint64_t accb = 0;
+            int      nb = 0, w = 0;
+            for (int i = 0; i < 32; i++) {
+                accb |= (uint64_t)((c[32 * h + i] & 15u) << 2) << nb;
+                nb += 6;
+                if (nb >= 32) { D[w++] = (uint32_t)accb; accb >>= 32; nb -= 32; }
+            }
+            v4u v = { D[0] | (D[4] & P), D[1] | (D[5] & Q), D[2] | (D[4] & R), D[3] | (D[5] & P) };
+            reinterpret_cast<v4u *>(dst)[h * 64 + lane] = v;
         }
     } else {
         constexpr uint32_t A = 0x10410410u, B = 0x04104104u, C = 0x41041041u;
@@ -551,11 +574,11 @@ template <int XB> __device__ __forceinline__ void store_native_lane(const uint8_
 }
 
 // Reference layout -> native layout on the device.  One thread per (row tile, K block, lane): it gathers its 64
-// codes bit piece by bit piece from the reference's segment arrays and writes its 10 or 12 native dwords.
+// codes bit piece by bit piece from the reference's segment arrays and writes its 8, 10 or 12 native dwords.
 __constant__ uint8_t kInvOrder4[8]  = { 4, 0, 6, 2, 5, 1, 7, 3 };
 __constant__ uint8_t kInvOrder2[16] = { 8, 0, 12, 4, 9, 1, 13, 5, 10, 2, 14, 6, 11, 3, 15, 7 };
 
-template <int XB>
+template <int FM>
 __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restrict__ native, const uint8_t *__restrict__ ref,
                                                              uint32_t M, uint32_t K, uint32_t units)
 {
@@ -565,9 +588,10 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
     const uint32_t R = blk / units, U = blk % units;
     const int      m = lane & 15, q = lane >> 4;
     const uint32_t row = R * 16 + m, tile = row >> 6, block = (row >> 4) & 3, rin = row & 15, g = rin & 7, rowhalf = rin >> 3;
-    // segment arrays: FP6 = [2-bit | 4-bit], FP5 = [1-bit | 4-bit]
+    // segment arrays: 6 bits = [2-bit | 4-bit], 5 bits = [1-bit | 4-bit], 4 bits = [4-bit]
+    constexpr int   bits = Fmt<FM>::bits;
     const uint32_t *seg_hi = reinterpret_cast<const uint32_t *>(ref);
-    const uint32_t *seg4   = reinterpret_cast<const uint32_t *>(ref + (size_t)M * K * (XB == 6 ? 2 : 1) / 8);
+    const uint32_t *seg4   = reinterpret_cast<const uint32_t *>(ref + (size_t)M * K * (bits - 4) / 8);
     uint8_t         c[64];
 #pragma unroll 1
     for (int s = 0; s < 8; s++) {
@@ -582,10 +606,10 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
                     uint32_t word = seg4[((size_t)(tile * (K / 16) + slice) * 4 + block) * 32 + l32];
                     code |= (word >> (28 - 4 * kInvOrder4[el])) & 15u;
                 }
-                if (XB == 6) { // 2-bit piece: q2 = block/2, pre = (block%2)*8 + el
+                if (bits == 6) { // 2-bit piece: q2 = block/2, pre = (block%2)*8 + el
                     uint32_t word = seg_hi[((size_t)(tile * (K / 16) + slice) * 2 + (block >> 1)) * 32 + l32];
                     code |= ((word >> (30 - 2 * kInvOrder2[(block & 1) * 8 + el])) & 3u) << 4;
-                } else { // 1-bit piece: q1 = 0, pre = block*8 + el; order_1 maps p -> pre, inverted arithmetically:
+                } else if (bits == 5) { // 1-bit piece: q1 = 0, pre = block*8 + el; order_1 maps p -> pre, inverted arithmetically:
                     // order_1[p]-1 = 4*(p%8) + {1,3,0,2}[p/8]  =>  p = 8*{2,0,3,1}[pre%4] + pre/4
                     uint32_t pre = block * 8 + el;
                     uint32_t p   = 8 * ((0x1302u >> (4 * (pre & 3))) & 3u) + (pre >> 2);
@@ -596,7 +620,7 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
             c[8 * s + j] = (uint8_t)code;
         }
     }
-    store_native_lane<XB>(c, native + (size_t)blk * Fmt<XB>::block_bytes, lane);
+    store_native_lane<FM>(c, native + (size_t)blk * Fmt<FM>::block_bytes, lane);
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -645,20 +669,20 @@ __global__ __launch_bounds__(256) void quant_row_scales(half_t *__restrict__ sca
 }
 
 // index (= magnitude bits of the code) of the representable magnitude nearest to a, 0 <= a <= max_value
-template <int XB> __device__ __forceinline__ uint32_t nearest_magnitude(double a)
+template <int FM> __device__ __forceinline__ uint32_t nearest_magnitude(double a)
 {
-    constexpr int bias = XB == 6 ? 3 : 1; // e3m2 / e2m2
+    constexpr int bias = Fmt<FM>::bias, MB = Fmt<FM>::man;
     int           e = a > 0.0 ? ilogb(a) : -1000;
     if (e < 1 - bias) e = 1 - bias;                        // subnormals use the spacing of the first binade
-    double   t = scalbn(a, 2 - e);                         // in units of the spacing 2^(e-2): [0,4) subnormal, [4,8) normal
+    double   t = scalbn(a, MB - e);                        // in units of the spacing 2^(e-MB): [0,2^MB) subnormal, [2^MB,2^(MB+1)) normal
     double   fl = floor(t), frac = t - fl;
-    uint32_t lo = (uint32_t)fl + (e > 1 - bias || fl >= 4.0 ? (uint32_t)(e + bias - 1) * 4u : 0u);
-    // (normal: index = (e+bias)*4 + (fl-4); subnormal: index = fl, and fl == 4 cannot happen there)
+    uint32_t lo = (uint32_t)fl + ((uint32_t)(e + bias - 1) << MB);
+    // (normal: index = (e+bias)*2^MB + (fl-2^MB); subnormal: e = 1-bias, so index = fl)
     if (frac > 0.5 || (frac == 0.5 && (lo & 1u))) lo += 1;
     return lo;
 }
 
-template <int XB, typename T>
+template <int FM, typename T>
 __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ native, const half_t *__restrict__ scales,
                                                       const T *__restrict__ Wf, uint32_t M, uint32_t K, uint32_t units, double max_value)
 {
@@ -680,31 +704,40 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
                 float  w = to_float<T>(p[k0 + j]);
                 double a = fabs((double)w / sc);
                 if (!(a <= max_value)) a = max_value; // clamps, and sends NaN to the maximum like a saturating cast
-                code = nearest_magnitude<XB>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (XB - 1));
+                code = nearest_magnitude<FM>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (Fmt<FM>::bits - 1));
             }
             c[8 * s + j] = (uint8_t)code;
         }
     }
-    store_native_lane<XB>(c, native + (size_t)blk * Fmt<XB>::block_bytes, lane);
+    store_native_lane<FM>(c, native + (size_t)blk * Fmt<FM>::block_bytes, lane);
 }
 
 // ------------------------------------------------------------------------------------------------ launch helpers
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
-template <int XB, int NT, int RT, int WAVES>
+// Calls fn with the format tag of a supported (E, M) as an integral constant.
+template <class Fn> inline int with_format(int E, int Mb, Fn &&fn)
+{
+    if (E == 3) return fn(std::integral_constant<int, 32>{});
+    if (Mb == 2) return fn(std::integral_constant<int, 22>{});
+    if (Mb == 3) return fn(std::integral_constant<int, 23>{});
+    return fn(std::integral_constant<int, 21>{});
+}
+
+template <int FM, int NT, int RT, int WAVES>
 int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
                   int splitK)
 {
     uint32_t units = (uint32_t)((K + 255) / 256);
     dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    hipLaunchKernelGGL((gemm_stream<XB, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
+    hipLaunchKernelGGL((gemm_stream<FM, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
                        static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M,
                        (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
     return (int)hipGetLastError();
 }
 
-template <int XB, int NT, int RT, int WR, int WK>
+template <int FM, int NT, int RT, int WR, int WK>
 int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K, int splitK)
 {
     constexpr int TN = NT * 16, TM = WR * RT * 16;
@@ -714,7 +747,7 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
     if (M % TM) return FP6MI_ERR_SHAPE;
     static bool attr_set = false; // idempotent, so a race between host threads is harmless
     if (!attr_set && lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<XB, NT, RT, WR, WK>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, NT, RT, WR, WK>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
@@ -722,7 +755,7 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
     uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
     size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
     if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
-    hipLaunchKernelGGL((gemm_tile<XB, NT, RT, WR, WK>), dim3((uint32_t)wgs), dim3(WR * WK * kWave), lds_bytes, st,
+    hipLaunchKernelGGL((gemm_tile<FM, NT, RT, WR, WK>), dim3((uint32_t)wgs), dim3(WR * WK * kWave), lds_bytes, st,
                        static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C),
                        ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
     return (int)hipGetLastError();
@@ -885,13 +918,13 @@ inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, i
     return c;
 }
 
-template <int XB>
+template <int FM>
 int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
                size_t K, int splitK)
 {
     if (c.kind == 0) {
 #define FP6MI_CASE(NT, RT, WV) \
-    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<XB, NT, RT, WV>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<FM, NT, RT, WV>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
         FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
@@ -902,7 +935,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
 #undef FP6MI_CASE
     } else if (c.kind == 1) {
 #define FP6MI_CASE(NT, RT, WR, WK) \
-    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<XB, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<FM, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
         FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
         FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1) FP6MI_CASE(4, 1, 4, 2) FP6MI_CASE(2, 1, 2, 4)
@@ -911,13 +944,13 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
     return FP6MI_ERR_SHAPE;
 }
 
-template <int XB>
+template <int FM>
 int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
                   int splitK, const LaunchCfg *forced)
 {
-    LaunchCfg c = forced ? *forced : pick_cfg(XB, M, N, K, splitK, 256);
+    LaunchCfg c = forced ? *forced : pick_cfg(Fmt<FM>::bits, M, N, K, splitK, 256);
     if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
-    int rc = launch_cfg<XB>(c, st, W, sc, B, C, ws, M, N, K, splitK);
+    int rc = launch_cfg<FM>(c, st, W, sc, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
     if (splitK > 1) {
         size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
@@ -938,7 +971,7 @@ const char *fp6mi_error_string(int code)
 {
     switch (code) {
     case FP6MI_OK: return "success";
-    case FP6MI_ERR_FORMAT: return "unsupported (E,M): only FP6_e3m2 (3,2) and FP5_e2m2 (2,2)";
+    case FP6MI_ERR_FORMAT: return "unsupported (E,M): only FP6_e3m2 (3,2), FP5_e2m2 (2,2), FP6_e2m3 (2,3) and FP4_e2m1 (2,1)";
     case FP6MI_ERR_SHAPE: return "unsupported shape: need M % 256 == 0 (64 for CPU packers, 16 for native packers), K % 64 == 0, N >= 1, distinct in/out";
     case FP6MI_ERR_NULL: return "a required pointer is NULL";
     case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
@@ -1029,7 +1062,7 @@ int fp6mi_linear_native(int E, int Mb, void *stream, const void *W, const void *
     int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
     if (rc != FP6MI_OK) return rc;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr);
+    return with_format(E, Mb, [&](auto fm) { return linear_native<decltype(fm)::value>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr); });
 }
 
 int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
@@ -1039,7 +1072,7 @@ int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const vo
     if (rc != FP6MI_OK) return rc;
     LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
-    return E == 3 ? linear_native<6>(st, W, sc, B, C, M, N, K, ws, splitK, &c) : linear_native<5>(st, W, sc, B, C, M, N, K, ws, splitK, &c);
+    return with_format(E, Mb, [&](auto fm) { return linear_native<decltype(fm)::value>(st, W, sc, B, C, M, N, K, ws, splitK, &c); });
 }
 
 int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, int *shape)
@@ -1048,7 +1081,7 @@ int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, 
     if (!shape) return FP6MI_ERR_NULL;
     if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
     if (splitK < 1) return FP6MI_ERR_SPLITK;
-    LaunchCfg c = pick_cfg(E == 3 ? 6 : 5, M, N, K, splitK, 256);
+    LaunchCfg c = pick_cfg(1 + E + Mb, M, N, K, splitK, 256);
     shape[0] = c.kind, shape[1] = c.nt, shape[2] = c.rt, shape[3] = c.wr, shape[4] = c.wk;
     return FP6MI_OK;
 }
@@ -1126,13 +1159,11 @@ int fp6mi_relayout_ref_to_native_gpu(int E, int Mb, void *stream, void *native, 
     size_t   blocks = (M / 16) * units;
     dim3     grid((uint32_t)((blocks + 3) / 4));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (E == 3)
-        hipLaunchKernelGGL(relayout_ref_to_native<6>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native), static_cast<const uint8_t *>(ref),
-                           (uint32_t)M, (uint32_t)K, units);
-    else
-        hipLaunchKernelGGL(relayout_ref_to_native<5>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native), static_cast<const uint8_t *>(ref),
-                           (uint32_t)M, (uint32_t)K, units);
-    return (int)hipGetLastError();
+    return with_format(E, Mb, [&](auto fm) {
+        hipLaunchKernelGGL(relayout_ref_to_native<decltype(fm)::value>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native),
+                           static_cast<const uint8_t *>(ref), (uint32_t)M, (uint32_t)K, units);
+        return (int)hipGetLastError();
+    });
 }
 
 int fp6mi_dequant_native_gpu(int E, int Mb, void *stream, void *out, const void *W, const void *sc, size_t M, size_t K)
@@ -1145,13 +1176,11 @@ int fp6mi_dequant_native_gpu(int E, int Mb, void *stream, void *out, const void 
     size_t   blocks = (M / 16) * units;
     dim3     grid((uint32_t)((blocks + 3) / 4));
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (E == 3)
-        hipLaunchKernelGGL(dequant_native<6>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
+    return with_format(E, Mb, [&](auto fm) {
+        hipLaunchKernelGGL(dequant_native<decltype(fm)::value>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
                            static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
-    else
-        hipLaunchKernelGGL(dequant_native<5>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
-                           static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
-    return (int)hipGetLastError();
+        return (int)hipGetLastError();
+    });
 }
 
 int fp6mi_quantize_native_gpu(int E, int Mb, void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K)
@@ -1164,29 +1193,25 @@ int fp6mi_quantize_native_gpu(int E, int Mb, void *stream, void *native, void *s
     const uint32_t units = (uint32_t)((K + 255) / 256);
     const size_t   blocks = (M / 16) * units;
     const dim3     grid_rows((uint32_t)((M + 3) / 4)), grid_blocks((uint32_t)((blocks + 3) / 4));
-    const double   max_value = E == 3 ? 28.0 : 7.0;
     hipStream_t    st = static_cast<hipStream_t>(stream);
     uint8_t       *nat = static_cast<uint8_t *>(native);
     half_t        *sc = static_cast<half_t *>(scales);
-#define FP6MI_QUANT(T)                                                                                                                    \
-    do {                                                                                                                                  \
-        hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, static_cast<const T *>(weights), (uint32_t)M, (uint32_t)K, \
-                           max_value);                                                                                                    \
-        if (E == 3)                                                                                                                       \
-            hipLaunchKernelGGL((quant_to_native<6, T>), grid_blocks, dim3(256), 0, st, nat, sc, static_cast<const T *>(weights),          \
-                               (uint32_t)M, (uint32_t)K, units, max_value);                                                               \
-        else                                                                                                                              \
-            hipLaunchKernelGGL((quant_to_native<5, T>), grid_blocks, dim3(256), 0, st, nat, sc, static_cast<const T *>(weights),          \
-                               (uint32_t)M, (uint32_t)K, units, max_value);                                                               \
-    } while (0)
-    if (dtype == 0)
-        FP6MI_QUANT(half_t);
-    else if (dtype == 1)
-        FP6MI_QUANT(bf16_t);
-    else
-        FP6MI_QUANT(float);
-#undef FP6MI_QUANT
-    return (int)hipGetLastError();
+    return with_format(E, Mb, [&](auto fm) {
+        constexpr int    FM = decltype(fm)::value;
+        constexpr double max_value = Fmt<FM>::max_value;
+        auto             run = [&](auto *typed) {
+            typedef std::remove_cv_t<std::remove_pointer_t<decltype(typed)>> T;
+            hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, typed, (uint32_t)M, (uint32_t)K, max_value);
+            hipLaunchKernelGGL((quant_to_native<FM, T>), grid_blocks, dim3(256), 0, st, nat, sc, typed, (uint32_t)M, (uint32_t)K, units, max_value);
+        };
+        if (dtype == 0)
+            run(static_cast<const half_t *>(weights));
+        else if (dtype == 1)
+            run(static_cast<const bf16_t *>(weights));
+        else
+            run(static_cast<const float *>(weights));
+        return (int)hipGetLastError();
+    });
 }
 
 } // extern "C"

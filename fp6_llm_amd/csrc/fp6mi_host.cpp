@@ -1,7 +1,7 @@
 // CPU half of the FPx linear-layer engine: reference-layout prepacking (bit-exact), dequantisation (bit-exact),
 // and the packers for the native gfx950 layout.  No GPU headers; built into the same shared library as the kernels.
 //
-// Formats: x = 1+E+M bit codes, (E,M) = (3,2) "FP6_e3m2" or (2,2) "FP5_e2m2".
+// Formats: x = 1+E+M bit codes, (E,M) = (3,2) "FP6_e3m2", (2,2) "FP5_e2m2", (2,3) "FP6_e2m3" or (2,1) "FP4_e2m1".
 // Raw tensor: row-major [M,K] codes, each row an MSB-first bitstream (code c = bits [c*x,(c+1)*x), bit 0 = MSB of
 // byte 0), the format defined by fp6_llm/csrc/utils/common.h:4-19 of the reference.
 #include "fp6mi_internal.h"
@@ -199,8 +199,8 @@ int unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K)
 
 // ------------------------------------------------------------------------------------------------ dequantisation
 //
-// value(code) = (-1)^s 2^(e-b) (1+m/4), e = 0: (-1)^s 2^(1-b) m/4, b = 2^(E-1)-1; every exponent is an ordinary value.
-// out = fp16_rn(value * float(scale)): the product of a 3-bit and an 11-bit significand is exact in FP32, so there is
+// value(code) = (-1)^s 2^(e-b) (1+m/2^M), e = 0: (-1)^s 2^(1-b) m/2^M, b = 2^(E-1)-1; every exponent is an ordinary value.
+// out = fp16_rn(value * float(scale)): the product of an at most 4-bit and an 11-bit significand is exact in FP32, so there is
 // one rounding, which is what utils/weight_dequant.h:30-43 of the reference computes.
 int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16)
 {
@@ -256,9 +256,22 @@ int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, c
 //   D5 = (S0 & A) | (S1 & B) | (((S2 & C) | (S3 & A) | (S4 & B)) << 1),   Dk = Sk & ~(its hole mask)
 // Eleven integer instructions rebuild the six dwords of 32 codes.  Lane dwords: string h has S0..S3 in dwords 4h..4h+3
 // and S4 in dword 8+h; dwords 0..7 sit at (d/4)*1024 + 16*l + 4*(d%4), dwords 8,9 at 2048 + 8*l + 4*(d-8).
-size_t native_block_bytes(int x) { return x == 6 ? 3072 : 2560; }
+//
+// FP6_e2m3 block (3072 B): the FP6_e3m2 block with e2m3 codes, the source format of v_cvt_scalef32_pk32_f16_fp6.
+//
+// FP4_e2m1 block (2048 B): again two strings of 32 six-bit fields per lane, each field = the FP4 code with two zeros appended
+// below its mantissa bit (s e1 e0 m 0 0): read as e2m3 that field is exactly the e2m1 value.  The two fixed-zero bits of the
+// 22 fields that start in D0..D3 are as many holes (44) as D4 and D5 have payload bits, at the same positions within a
+// dword, so storage keeps four dwords S0..S3 per string and no bit has to shift:
+//   S0 = D0 | (D4 & P)   S1 = D1 | (D5 & Q)   S2 = D2 | (D4 & R)   S3 = D3 | (D5 & P)
+//   P = 0xC30C30C3 (bit pairs 0,6,..,30)   Q = 0x30C30C30 (pairs 4,10,..,28)   R = 0x0C30C30C (pairs 2,8,..,26)
+//   D4 = (S0 & P) | (S2 & R),   D5 = (S1 & Q) | (S3 & P),   D0 = S0 & ~P,  D1 = S1 & ~Q,  D2 = S2 & ~R,  D3 = S3 & ~P
+// Lane dwords: string h has S0..S3 in dwords 4h..4h+3 at (d/4)*1024 + 16*l + 4*(d%4).
+size_t native_block_bytes(int x) { return x == 6 ? 3072 : x == 5 ? 2560 : 2048; }
+static inline int native_lane_dwords(int x) { return x == 6 ? 12 : x == 5 ? 10 : 8; }
 
 static const uint32_t kHoleA = 0x10410410u, kHoleB = 0x04104104u, kHoleC = 0x41041041u;
+static const uint32_t kPairP = 0xC30C30C3u, kPairQ = 0x30C30C30u, kPairR = 0x0C30C30Cu;
 
 // 32 six-bit fields -> six dwords (little-endian bit string), and back
 static void fields_to_dwords(const uint8_t f[32], uint32_t o[6])
@@ -283,7 +296,7 @@ static void dwords_to_fields(const uint32_t o[6], uint8_t f[32])
 
 static inline size_t native_dword_offset(int x, int lane, int d)
 {
-    if (x == 6 || d < 8) return (size_t)(d / 4) * 1024 + (size_t)lane * 16 + (size_t)(d % 4) * 4;
+    if (x != 5 || d < 8) return (size_t)(d / 4) * 1024 + (size_t)lane * 16 + (size_t)(d % 4) * 4;
     return 2048 + (size_t)lane * 8 + (size_t)(d - 8) * 4;
 }
 
@@ -292,6 +305,15 @@ static void native_pack_lane(int x, const uint8_t c[64], uint32_t d[12])
     for (int h = 0; h < 2; h++) {
         if (x == 6) {
             fields_to_dwords(c + 32 * h, d + 6 * h);
+        } else if (x == 4) {
+            uint8_t  f[32];
+            uint32_t D[6];
+            for (int i = 0; i < 32; i++) f[i] = (uint8_t)((c[32 * h + i] & 15u) << 2);
+            fields_to_dwords(f, D);
+            d[4 * h + 0] = D[0] | (D[4] & kPairP);
+            d[4 * h + 1] = D[1] | (D[5] & kPairQ);
+            d[4 * h + 2] = D[2] | (D[4] & kPairR);
+            d[4 * h + 3] = D[3] | (D[5] & kPairP);
         } else {
             uint8_t  f[32];
             uint32_t D[6];
@@ -311,6 +333,12 @@ static void native_unpack_lane(int x, const uint32_t d[12], uint8_t c[64])
     for (int h = 0; h < 2; h++) {
         if (x == 6) {
             dwords_to_fields(d + 6 * h, c + 32 * h);
+        } else if (x == 4) {
+            const uint32_t S0 = d[4 * h], S1 = d[4 * h + 1], S2 = d[4 * h + 2], S3 = d[4 * h + 3];
+            uint32_t       D[6] = { S0 & ~kPairP, S1 & ~kPairQ, S2 & ~kPairR, S3 & ~kPairP, (S0 & kPairP) | (S2 & kPairR), (S1 & kPairQ) | (S3 & kPairP) };
+            uint8_t        f[32];
+            dwords_to_fields(D, f);
+            for (int i = 0; i < 32; i++) c[32 * h + i] = (uint8_t)(f[i] >> 2);
         } else {
             const uint32_t S0 = d[4 * h], S1 = d[4 * h + 1], S2 = d[4 * h + 2], S3 = d[4 * h + 3], S4 = d[8 + h];
             uint32_t       D[6] = { S0 & ~kHoleA, S1 & ~kHoleB, S2 & ~kHoleC, S3 & ~kHoleA, S4 & ~kHoleB,
@@ -332,7 +360,7 @@ size_t native_bytes(int E, int Mb, size_t M, size_t K)
 static void native_pack_rowtile(int x, size_t K, const uint8_t *codes, uint8_t *tile_out)
 {
     size_t units = (K + 255) / 256, bb = native_block_bytes(x);
-    int    nd = (x == 6) ? 12 : 10;
+    int    nd = native_lane_dwords(x);
     for (size_t U = 0; U < units; U++)
         for (int lane = 0; lane < 64; lane++) {
             int     m = lane & 15, q = lane >> 4;
@@ -350,7 +378,7 @@ static void native_pack_rowtile(int x, size_t K, const uint8_t *codes, uint8_t *
 static void native_unpack_rowtile(int x, size_t K, const uint8_t *tile_in, uint8_t *codes)
 {
     size_t units = (K + 255) / 256, bb = native_block_bytes(x);
-    int    nd = (x == 6) ? 12 : 10;
+    int    nd = native_lane_dwords(x);
     for (size_t U = 0; U < units; U++)
         for (int lane = 0; lane < 64; lane++) {
             int      m = lane & 15, q = lane >> 4;

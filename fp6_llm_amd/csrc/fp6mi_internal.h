@@ -10,7 +10,8 @@
 
 namespace fp6mi {
 
-inline bool supported(int E, int Mbits) { return Mbits == 2 && (E == 2 || E == 3); }
+// FP6_e3m2 and FP5_e2m2 (the formats of the reference's entry points), FP6_e2m3 and FP4_e2m1 (through the same paths)
+inline bool supported(int E, int Mbits) { return (E == 3 && Mbits == 2) || (E == 2 && (Mbits == 1 || Mbits == 2 || Mbits == 3)); }
 
 // fp6mi_host.cpp
 int    prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K);

@@ -39,7 +39,8 @@ at::Tensor workspace_for(const at::Device &dev, void *stream, int64_t floats)
 at::Tensor linear_forward_native(int64_t E, int64_t Mb, const at::Tensor &in_feats, const at::Tensor &native_weight, const at::Tensor &scales,
                                  int64_t OC, int64_t splitK, const c10::optional<at::Tensor> &out_opt, const c10::optional<at::Tensor> &ws_opt)
 {
-    if (!((E == 3 || E == 2) && Mb == 2)) bad("unsupported format: EXPONENT=" + std::to_string(E) + ", MANTISSA=" + std::to_string(Mb) + " (only e3m2 and e2m2)");
+    const bool known = (E == 3 && Mb == 2) || (E == 2 && Mb >= 1 && Mb <= 3);
+    if (!known) bad("unsupported format: EXPONENT=" + std::to_string(E) + ", MANTISSA=" + std::to_string(Mb) + " (only e3m2, e2m2, e2m3 and e2m1)");
     if (in_feats.scalar_type() != at::kHalf || in_feats.dim() != 2) bad("in_feats must be a 2-D float16 tensor [B, IC]");
     if (!in_feats.is_cuda()) bad("in_feats must be on the GPU");
     const at::Device dev = in_feats.device();
@@ -47,7 +48,7 @@ at::Tensor linear_forward_native(int64_t E, int64_t Mb, const at::Tensor &in_fea
     if (scales.scalar_type() != at::kHalf || scales.numel() != OC) bad("scales must be float16 [OC]");
     const int64_t B = in_feats.size(0), IC = in_feats.size(1);
     if (OC % 256 != 0 || IC % 64 != 0 || B < 1) bad("need OC % 256 == 0, IC % 64 == 0, B >= 1");
-    const int64_t want = (OC / 16) * ((IC + 255) / 256) * (E == 3 ? 3072 : 2560);
+    const int64_t want = (int64_t)fp6mi_native_bytes((int)E, (int)Mb, (size_t)OC, (size_t)IC);
     if ((int64_t)native_weight.numel() * (int64_t)native_weight.element_size() != want) bad("native_weight has the wrong size for OC and IC");
     if (splitK < 1) bad("splitK must be >= 1");
     if (!native_weight.is_contiguous()) bad("native_weight must be contiguous");

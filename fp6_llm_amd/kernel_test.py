@@ -72,7 +72,7 @@ def main(argv=None):
     ap.add_argument("--BS", type=int, default=32, help="batch size")
     ap.add_argument("--splitK", type=int, default=0, help="split of the K dimension; 0 = the engine's heuristic")
     ap.add_argument("--EXP", type=int, default=3, choices=(2, 3), help="exponent bits")
-    ap.add_argument("--MAN", type=int, default=2, choices=(2,), help="mantissa bits")
+    ap.add_argument("--MAN", type=int, default=2, choices=(1, 2, 3), help="mantissa bits (e3m2, e2m2, e2m3 and e2m1 exist)")
     ap.add_argument("--repeat", type=int, default=1000)
     a = ap.parse_args(argv)
     run(a.OC, a.IC, a.BS, a.splitK, a.EXP, a.MAN, a.repeat)

@@ -1,14 +1,18 @@
 """FP16/FP32 -> FPx quantizer with per-row absmax scales, and raw-tensor packing.
 
 The reference ships only a truncating FP16->FP6 cast that is not wired into any API (fp6_llm/csrc/utils/weight_quant.h:9-105,
-"To be used in the future"); this one rounds to nearest, ties to even, clamps at the format maximum and covers e2m2 too.
+"To be used in the future"); this one rounds to nearest, ties to even, clamps at the format maximum and covers every format of the
+engine (e3m2, e2m2, e2m3, e2m1).
 It is the step before the linear-layer path: it produces the raw int32 tensor that weight_prepacking*_cpu consumes.
 """
 import numpy as np
 
 
+FORMATS = ((3, 2), (2, 2), (2, 3), (2, 1))   # FP6_e3m2, FP5_e2m2, FP6_e2m3, FP4_e2m1
+
+
 def _check(E, M):
-    if (E, M) not in ((3, 2), (2, 2)):
+    if (E, M) not in FORMATS:
         raise ValueError("unsupported format e%dm%d" % (E, M))
     return 1 + E + M
 
@@ -69,6 +73,8 @@ def pack_raw(codes, E=3, M=2):
         out[:, :, 0] = (q[:, :, 0] << 2) | (q[:, :, 1] >> 4)
         out[:, :, 1] = (q[:, :, 1] << 4) | (q[:, :, 2] >> 2)
         out[:, :, 2] = (q[:, :, 2] << 6) | q[:, :, 3]
+    elif x == 4:  # 2 codes -> 1 byte
+        out = (c[:, 0::2] << 4) | c[:, 1::2]
     else:        # 8 codes -> 5 bytes
         q = c.reshape(c.shape[0], -1, 8)
         out = np.empty((c.shape[0], q.shape[1], 5), dtype=np.uint8)

@@ -27,6 +27,7 @@ STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4)]                      # two 16-c
 TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
         (1, 8, 2, 8, 1)]
 SPLITS = (1, 2, 4, 8)
+FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit width
 
 # every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip); the candidates above are the ones that
 # ever came within 3 % of the best in exhaustive sweeps
@@ -129,7 +130,7 @@ class Bench:
 
 
 def sweep(args):
-    E, M = (3, 2) if args.format == 6 else (2, 2)
+    E, M = FORMAT_OF_BITS[args.format]
     Ms = [int(v) for v in args.m.split(",")] if args.m else GRID_M
     Ks = [int(v) for v in args.k.split(",")] if args.k else GRID_K
     Ns = [int(v) for v in args.n.split(",")] if args.n else GRID_N_SMALL + GRID_N_LARGE
@@ -179,7 +180,8 @@ def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
     s = sub.add_parser("sweep")
-    s.add_argument("--format", type=int, choices=(5, 6), default=6)
+    s.add_argument("--format", type=int, choices=sorted(FORMAT_OF_BITS), default=6,
+                   help="bit width: 6 = e3m2 (e2m3 streams the same bytes and shares its table), 5 = e2m2, 4 = e2m1")
     s.add_argument("--out", required=True)
     s.add_argument("--append", action="store_true")
     s.add_argument("--m", default="")

@@ -7,7 +7,10 @@
  * (paths relative to that repository).
  *
  * Conventions (same as the reference, fp6_llm/csrc/fp6_linear.cu:149-159):
- *   M = OC (weight rows), K = IC, N = batch.  Weights are x = 1+E+M bit codes, (E,M) in {(3,2), (2,2)}.
+ *   M = OC (weight rows), K = IC, N = batch.  Weights are x = 1+E+M bit codes: (E,M) = (3,2) FP6_e3m2 and (2,2) FP5_e2m2,
+ *   the formats the reference's entry points admit (fp6_llm/csrc/fp6_linear.cu:133-138), and through the same entry points
+ *   (2,3) FP6_e2m3 and (2,1) FP4_e2m1, which the reference's templates allow (utils/weight_prepacking.h:43) but its
+ *   dispatchers reject.
  *   "raw" weights     : row-major [M,K] codes, per-row MSB-first bitstream, M*K*x/8 bytes.
  *   "ref" layout      : the reference's prepacked layout (utils/weight_prepacking.h:118-196), same byte count.
  *   "native" layout   : this engine's gfx950 layout, fp6mi_native_bytes() bytes (K padded to 256).
@@ -28,7 +31,7 @@ extern "C" {
 #endif
 
 #define FP6MI_OK 0
-#define FP6MI_ERR_FORMAT (-1)    /* (E,M) is not (3,2) or (2,2)             */
+#define FP6MI_ERR_FORMAT (-1)    /* (E,M) is not (3,2), (2,2), (2,3), (2,1) */
 #define FP6MI_ERR_SHAPE (-2)     /* M % 256, K % 64, N > 0 or size overflow */
 #define FP6MI_ERR_NULL (-3)      /* a required pointer is NULL              */
 #define FP6MI_ERR_WORKSPACE (-4) /* splitK > 1 without a workspace          */

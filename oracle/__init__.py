@@ -77,6 +77,9 @@ def ref_lib():
         R.ref_weight_matrix_prepacking_fp_eXmY.restype = None
         R.ref_weight_matrix_prepacking.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
         R.ref_weight_matrix_prepacking.restype = None
+        R.ref_weight_matrix_prepacking_x_bit.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p,
+                                                         ctypes.c_void_p, ctypes.c_size_t, ctypes.c_size_t]
+        R.ref_weight_matrix_prepacking_x_bit.restype = ctypes.c_int
         _REF = R
     return _REF
 
@@ -192,7 +195,10 @@ def ref_prepack(raw, E=3, M=2):
     padded = np.zeros(b.size + 64, dtype=np.uint8)
     padded[: b.size] = b.reshape(-1)
     out = np.zeros(b.size + 64, dtype=np.uint8)
-    R.ref_weight_matrix_prepacking_fp_eXmY(E, M, _ptr(out), _ptr(padded), rows, K)
+    if (E, M) in ((3, 2), (2, 2)):
+        R.ref_weight_matrix_prepacking_fp_eXmY(E, M, _ptr(out), _ptr(padded), rows, K)
+    elif R.ref_weight_matrix_prepacking_x_bit(E, M, _ptr(out), _ptr(padded), rows, K) != 0:  # the template, other (E,M)
+        raise ValueError("no instantiation of the reference's prepacking template for E=%d M=%d" % (E, M))
     return out[: b.size].reshape(b.shape).copy()
 
 

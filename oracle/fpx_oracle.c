@@ -107,7 +107,11 @@ static uint8_t orc_left_aligned_code(const uint8_t *bytes, size_t nbytes, size_t
     return (uint8_t)(top & (uint8_t)(0xff00u >> x));
 }
 
-static int orc_supported(int E, int M) { return (M == 2) && (E == 2 || E == 3); }
+/* e3m2 and e2m2 are the formats the reference's entry points admit (utils/weight_prepacking.h:204-211, fp6_linear.cu:133-138).
+ * e2m3 and e2m1 go through the same templates of the reference (any 1+E+M < 8, utils/weight_prepacking.h:43); for them the
+ * prepacker is pinned against the reference's template instantiated for those (E,M), the dequantizer against the format
+ * definition only. */
+static int orc_supported(int E, int M) { return (E == 3 && M == 2) || (E == 2 && (M == 1 || M == 2 || M == 3)); }
 
 /* codes[r*K + c] = right-aligned x-bit code */
 int orc_unpack_codes(int E, int M, uint8_t *codes, const uint8_t *raw, size_t rows, size_t K)

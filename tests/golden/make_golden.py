@@ -6,7 +6,9 @@ Run in the build container only (it needs /root/reference to have been compiled 
 
 What it writes
   prepack_<fmt>_<OC>x<IC>.npz : raw int32 weights (deterministic codes) and the bytes the reference's
-                                weight_matrix_prepacking_fp_eXmY (utils/weight_prepacking.h:204-211) produced for them.
+                                weight_matrix_prepacking_fp_eXmY (utils/weight_prepacking.h:204-211) produced for them;
+                                for e2m3 and e2m1, which that dispatcher does not admit, the bytes of the template it
+                                dispatches to (weight_matrix_prepacking_x_bit, :118-196) instantiated for that (E, M).
   prepack_hashes.json         : SHA-256 of raw and reference-prepacked buffers at benchmark sizes
                                 (config 1: 256x1024, config 2: 4096x4096), whose inputs any machine regenerates from
                                 fp6_llm_amd.synth.uniform_codes(seed, ...).
@@ -27,7 +29,7 @@ import oracle  # noqa: E402
 from fp6_llm_amd import quant, synth  # noqa: E402
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-FMT = {"e3m2": (3, 2), "e2m2": (2, 2)}
+FMT = {"e3m2": (3, 2), "e2m2": (2, 2), "e2m3": (2, 3), "e2m1": (2, 1)}
 
 
 def main():

@@ -17,7 +17,7 @@ from fp6_llm_amd import _lib, quant, synth
 
 pytestmark = pytest.mark.gpu
 
-FORMATS = [(3, 2), (2, 2)]
+FORMATS = [(3, 2), (2, 2), (2, 3), (2, 1)]
 TOL_MAX_REL = 1e-2
 TOL_MEAN_REL = 2e-3
 DEV = "cuda:0"
@@ -161,10 +161,13 @@ def test_unsupported_launch_shape_is_rejected():
 def test_known_answers(E, M):
     """All-ones weights/activations/scales => every output = IC (tests/python/kernel_test_fpx.py:88-131);
     one-hot activations => a column of the dequantized weights, bit for bit; zero scale => zeros."""
-    ones = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2): [806142768, 3274706115, 214118412]}[(E, M)]
+    ones = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2): [806142768, 3274706115, 214118412]}
     OC, IC = 256, 1024
-    words = np.array(ones, dtype=np.uint32)
-    raw = np.tile(words, (OC, IC * (1 + E + M) // 32 // len(words))).view(np.int32)
+    if (E, M) in ones:
+        words = np.array(ones[(E, M)], dtype=np.uint32)
+        raw = np.tile(words, (OC, IC * (1 + E + M) // 32 // len(words))).view(np.int32)
+    else:   # formats outside the reference's tests: the code of 1.0 (exponent field = bias = 1, mantissa 0) everywhere
+        raw = quant.pack_raw(np.full((OC, IC), 1 << M, np.uint8), E, M)
     native, scd, xd = upload(raw, np.ones(OC, np.float16), np.ones((8, IC), np.float16), E, M)
     assert (gemm_capi(E, M, native, scd, xd, OC) == np.float16(IC)).all()
 

@@ -15,7 +15,8 @@ import oracle
 import fp6_llm_amd as fp6
 from fp6_llm_amd import _lib, quant, synth
 
-FORMATS = [(3, 2), (2, 2)]
+FORMATS = [(3, 2), (2, 2), (2, 3), (2, 1)]
+BLOCK_BYTES = {6: 3072, 5: 2560, 4: 2048}   # native layout: bytes of a 16-row x 256-column block, by bit width
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
@@ -37,7 +38,7 @@ def test_library_exports_every_declared_symbol():
 
 def test_golden_prepack_fixtures(golden_dir):
     for f in sorted(glob.glob(os.path.join(golden_dir, "prepack_e*_*.npz"))):
-        E, M = (3, 2) if "e3m2" in f else (2, 2)
+        E, M = (int(v) for v in re.search(r"prepack_e(\d)m(\d)_", f).groups())
         z = np.load(f)
         raw = np.ascontiguousarray(z["raw"])
         OC, IC = raw.shape[0], raw.shape[1] * 32 // (1 + E + M)
@@ -69,7 +70,7 @@ def test_prepack_dequant_native_against_oracle(E, M, OC, IC):
     assert (dq.view(np.uint16) == oracle.dequant(raw, sc, E, M).view(np.uint16)).all()
     # native layout: same bits by both routes, and a lossless round trip
     nat = fp6.weight_prepacking_native_cpu(E, M, t)
-    assert nat.numel() * 4 == fp6.native_bytes(E, M, OC, IC) == (OC // 16) * ((IC + 255) // 256) * (3072 if E == 3 else 2560)
+    assert nat.numel() * 4 == fp6.native_bytes(E, M, OC, IC) == (OC // 16) * ((IC + 255) // 256) * BLOCK_BYTES[1 + E + M]
     assert torch.equal(nat, fp6.to_native(packed, E, M))
     L = _lib.lib()
     back = np.empty_like(raw)
@@ -93,12 +94,23 @@ def test_native_fp6_lane_image_is_the_hardware_operand(E, M):
     OC, IC = 32, 512
     codes = synth.uniform_codes(42, OC, IC, E, M)
     nat = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))).numpy().view(np.uint32)
-    bb = (3072 if E == 3 else 2560) // 4
+    bb = BLOCK_BYTES[x] // 4
     for (R, U, lane) in [(0, 0, 0), (1, 1, 37), (0, 1, 63), (1, 0, 16)]:
         m, q = lane % 16, lane // 16
         blk = nat[(R * 2 + U) * bb:(R * 2 + U + 1) * bb]
         want = [codes[16 * R + m, 256 * U + 32 * s + 8 * q + j] for s in range(8) for j in range(8)]
-        if E == 3:
+        if x == 4:
+            d = [blk[(i // 4) * 256 + lane * 4 + i % 4] for i in range(8)]
+            # four stored dwords per string; dwords five and six of the 6-bit string sit in the two fixed-zero low bits of the fields
+            P, Q, R = 0xC30C30C3, 0x30C30C30, 0x0C30C30C
+            for h in range(2):
+                S = [int(d[4 * h + k]) for k in range(4)]
+                D = [S[0] & ~P, S[1] & ~Q, S[2] & ~R, S[3] & ~P, (S[0] & P) | (S[2] & R), (S[1] & Q) | (S[3] & P)]
+                big = sum(D[w] << (32 * w) for w in range(6))
+                fields = [(big >> (6 * i)) & 63 for i in range(32)]
+                assert all(f & 3 == 0 for f in fields)                 # the two bits appended below the mantissa
+                assert [f >> 2 for f in fields] == [int(v) for v in want[32 * h:32 * h + 32]]
+        elif x == 6:
             d = [blk[(i // 4) * 256 + lane * 4 + i % 4] for i in range(12)]
             for h in range(2):
                 big = sum(int(d[6 * h + w]) << (32 * w) for w in range(6))
@@ -221,7 +233,7 @@ def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it()
     L = _lib.lib()
     shape = (ctypes.c_int * 5)()
     for xb, m256, k64, n, cells in entries:
-        E = 3 if int(xb) == 6 else 2
+        E, Mb = {6: (3, 2), 5: (2, 2), 4: (2, 1)}[int(xb)]
         OC, IC, BS = int(m256) * 256, int(k64) * 64, int(n)
         for i, cell in enumerate(re.findall(r"\{([\d,]+)\}", cells)):
             v = tuple(int(t) for t in cell.split(","))
@@ -229,12 +241,12 @@ def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it()
                 continue
             assert v[:5] in compiled, (xb, OC, IC, BS, v)
             assert OC % tune.tile_rows(v[:5]) == 0
-            assert L.fp6mi_query_launch(E, 2, OC, BS, IC, 1 << i, shape) == 0
+            assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, 1 << i, shape) == 0
             assert tuple(shape) == v[:5], (xb, OC, IC, BS, 1 << i, tuple(shape), v)
     # any legal problem gets a compiled shape that divides its rows, measured neighbour or not
     for (OC, IC, BS, sk) in [(256, 64, 1, 1), (768, 1088, 3, 2), (4352, 4160, 8, 1), (9984, 3008, 40, 3), (65536, 16384, 700, 1), (512, 64, 17, 1)]:
-        for E in (3, 2):
-            assert L.fp6mi_query_launch(E, 2, OC, BS, IC, sk, shape) == 0
+        for (E, Mb) in FORMATS:
+            assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, sk, shape) == 0
             assert tuple(shape) in compiled and OC % tune.tile_rows(tuple(shape)) == 0, (OC, IC, BS, sk, tuple(shape))
     assert L.fp6mi_query_launch(3, 2, 100, 1, 64, 1, shape) == -2 and L.fp6mi_query_launch(4, 3, 256, 1, 64, 1, shape) == -1
 
@@ -300,7 +312,7 @@ def test_module_construction_routes_agree():
 def test_fused_layers_are_the_concatenation():
     """Fusing layers over one input = quantizing the row-concatenated weight: native tiles are stored row tile after row tile."""
     from fp6_llm_amd import module
-    for (E, M) in ((3, 2), (2, 2)):
+    for (E, M) in FORMATS:
         ws = [torch.from_numpy(synth.normal(61 + i, (oc, 320))).float() for i, oc in enumerate((256, 512, 256))]
         bs = [torch.from_numpy(synth.normal(71 + i, (w.shape[0],))).half() for i, w in enumerate(ws)]
         parts = [module.FPxLinear.from_float(w, E, M, bias=b) for w, b in zip(ws, bs)]
@@ -322,6 +334,14 @@ def test_e2m2_code_read_as_e3m2_is_a_quarter_of_its_value():
         assert v6[field] * 4.0 == v5[code] and np.signbit(v6[field]) == np.signbit(v5[code])
 
 
+def test_e2m1_code_with_two_zeros_appended_is_the_e2m3_code_of_its_value():
+    """What the FP4 native layout relies on: an e2m1 code shifted left by two bits is the e2m3 code of the same value, for all
+    16 codes (the subnormal and the signed zeros included)."""
+    v4, v6 = oracle.value_table(2, 1), oracle.value_table(2, 3)
+    for code in range(16):
+        assert v6[code << 2] == v4[code] and np.signbit(v6[code << 2]) == np.signbit(v4[code])
+
+
 def test_bench_refuses_more_than_one_gpu_and_lists_the_benchmark_configurations():
     import subprocess
     import sys
@@ -333,7 +353,7 @@ def test_bench_refuses_more_than_one_gpu_and_lists_the_benchmark_configurations(
     assert bench.WORKLOADS[bench.HEADLINE] == (3, 2, 4096, 4096, 8)
     # every shape of the five benchmark configurations is a workload: 4096^2 at 1/8/16, the two 7B MLP shapes at 8/32, the three
     # 70B shapes at 32, and 8192^2 at ten batch sizes in both formats
-    assert len(bench.WORKLOADS) == 3 + 4 + 3 + 20
+    assert len([w for w in bench.WORKLOADS if w.startswith(("fp6_", "fp5_"))]) == 3 + 4 + 3 + 20
     assert bench.weight_bytes(3, 2, 4096, 4096) == 12582912 and bench.algorithmic_bytes(3, 2, 4096, 4096, 8) == 12722176
 
 

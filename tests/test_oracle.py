@@ -8,6 +8,7 @@ import glob
 import hashlib
 import json
 import os
+import re
 import struct
 from fractions import Fraction
 
@@ -17,12 +18,15 @@ import pytest
 import oracle
 from fp6_llm_amd import quant, synth
 
-FORMATS = [(3, 2), (2, 2)]
+FORMATS = [(3, 2), (2, 2), (2, 3), (2, 1)]
+CODE_OF_ONE = {(3, 2): 0b001100, (2, 2): 0b00100, (2, 3): 0b001000, (2, 1): 0b0010}   # sign 0, exponent = bias, mantissa 0
 # "all weights = 1.0" bit patterns quoted in the reference: tests/python/kernel_test_fpx.py:88-107 (FP5_e2m2) and :110-131 (FP6_e3m2)
 ONES = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2): [806142768, 3274706115, 214118412]}
 
 
 def _ones_raw(E, M, OC, IC):
+    if (E, M) not in ONES:   # formats the reference's tests do not cover: the same tensor from the format definition
+        return quant.pack_raw(np.full((OC, IC), CODE_OF_ONE[(E, M)], np.uint8), E, M)
     words = np.array(ONES[(E, M)], dtype=np.uint32)
     reps = IC // (32 * len(words) // (1 + E + M))
     return np.tile(words, (OC, reps)).view(np.int32)
@@ -34,7 +38,7 @@ def test_all_ones_pattern_decodes_to_the_code_of_one(E, M):
     # 1.0 = sign 0, exponent = bias, mantissa 0: e3m2 -> 0 011 00 = 12, e2m2 -> 0 01 00 = 4 (kernel_test_fpx.py:102,125)
     raw = _ones_raw(E, M, 64, 128)
     codes = oracle.unpack_codes(raw, E, M)
-    assert set(np.unique(codes)) == {12 if E == 3 else 4}
+    assert set(np.unique(codes)) == {CODE_OF_ONE[(E, M)]}
     assert (oracle.raw_to_codes(raw, E, M) == codes).all()
 
 
@@ -54,9 +58,9 @@ def test_bitstream_is_msb_first(E, M):
 # ------------------------------------------------------------------------------------------------ prepacking
 def test_golden_prepack_fixtures(golden_dir):
     files = sorted(glob.glob(os.path.join(golden_dir, "prepack_e*_*.npz")))
-    assert len(files) == 6
+    assert len(files) == 12
     for f in files:
-        E, M = (3, 2) if "e3m2" in f else (2, 2)
+        E, M = (int(v) for v in re.search(r"prepack_e(\d)m(\d)_", f).groups())
         z = np.load(f)
         got = oracle.prepack(z["raw"], E, M)
         assert got.tobytes() == z["packed"].tobytes(), f
@@ -95,12 +99,13 @@ def test_prepack_closed_form_index_map(E, M):
 
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_prepack_all_ones_known_answer(E, M):
-    # 1.0 splits into an all-zero high segment and the nibble 1100 (e3m2) / 0100 (e2m2) in every 4-bit fragment
+    # 1.0 splits into an all-zero high segment (if any) and the low nibble of its code (1100 for e3m2, 0100 for e2m2,
+    # 1000 for e2m3, 0010 for e2m1) in every 4-bit fragment
     raw = _ones_raw(E, M, 64, 128)
     words = oracle.prepack(raw, E, M).view(np.uint32).reshape(-1)
-    hi_words = 64 * 128 * (2 if E == 3 else 1) // 32
+    hi_words = 64 * 128 * (1 + E + M - 4) // 32
     assert (words[:hi_words] == 0).all()
-    assert (words[hi_words:] == (0xCCCCCCCC if E == 3 else 0x44444444)).all()
+    assert (words[hi_words:] == (CODE_OF_ONE[(E, M)] & 15) * 0x11111111).all()
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
@@ -143,10 +148,14 @@ def _half_bits_of_fraction(v):
 def test_format_constants(E, M):
     tab = oracle.value_table(E, M)
     x = 1 + E + M
-    if E == 3:  # utils/weight_quant.h:22-25: max 28, smallest subnormal 0.0625
+    if (E, M) == (3, 2):  # utils/weight_quant.h:22-25: max 28, smallest subnormal 0.0625
         assert tab[0b011111] == 28.0 and tab[0b000001] == 0.0625 and tab[0b001100] == 1.0
-    else:
+    elif (E, M) == (2, 2):
         assert tab[0b01111] == 7.0 and tab[0b00001] == 0.25 and tab[0b00100] == 1.0
+    elif (E, M) == (2, 3):  # OCP Microscaling Formats (MX) v1.0, table 3: FP6 E2M3 max normal 7.5, min subnormal 0.125
+        assert tab[0b011111] == 7.5 and tab[0b000001] == 0.125 and tab[0b001000] == 1.0 and tab[0b000111] == 0.875
+    else:                   # same table: FP4 E2M1 max normal 6.0, min subnormal 0.5; the eight magnitudes of the format
+        assert list(tab[:8]) == [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
     assert (tab[(1 << (x - 1)):] == -tab[: (1 << (x - 1))]).all()
     assert np.signbit(tab[1 << (x - 1)]) and tab[1 << (x - 1)] == 0.0   # negative zero exists
     assert np.isfinite(tab).all()                                       # exponent all-ones is an ordinary value
