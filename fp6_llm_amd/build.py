@@ -6,7 +6,11 @@ import sys
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SOURCES = [os.path.join(HERE, "csrc", "fp6mi_host.cpp"), os.path.join(HERE, "csrc", "fp6mi_gemm.hip")]
+# (source, object name, extra flags): the kernel file is compiled once per weight format (tag = 10*E + M), the objects in parallel
+FORMAT_TAGS = (32, 22, 23, 21)
+UNITS = [("fp6mi_host.cpp", "fp6mi_host.o", []), ("fp6mi_api.hip", "fp6mi_api.o", [])] + \
+        [("fp6mi_gemm.hip", "fp6mi_gemm_%d.o" % t, ["-DFP6MI_FORMAT=%d" % t]) for t in FORMAT_TAGS]
+OBJ_DIR = os.path.join(HERE, "csrc", "obj")
 OUTPUT = os.path.join(HERE, "libfp6mi.so")
 # measurement aid for the benchmark (a read-only streaming kernel); not linked into the engine
 PROBE_SOURCES = [os.path.join(HERE, "csrc", "stream_probe.hip")]
@@ -20,18 +24,39 @@ def hipcc_path():
     raise RuntimeError("hipcc not found; the FPx engine cannot be built without the ROCm compiler")
 
 
-def _compile(sources, output, verbose):
-    cmd = [hipcc_path(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-shared",
+def _hipcc(args, what, verbose):
+    cmd = [hipcc_path(), "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
            # packed FP32 VALU forms are kept out of the generated code on this hardware pool
            "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           "-I" + os.path.join(ROOT, "include")] + sources + ["-o", output + ".tmp"]
+           "-I" + os.path.join(ROOT, "include")] + args
     res = subprocess.run(cmd, capture_output=True, text=True)
     if verbose or res.returncode != 0:
-        sys.stderr.write(res.stdout + res.stderr)
+        sys.stderr.write("\n".join(l for l in (res.stdout + res.stderr).splitlines() if "packed-fp32-ops" not in l) + "\n")
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed building " + os.path.basename(output))
+        raise RuntimeError("hipcc failed building " + what)
+
+
+def _compile(sources, output, verbose):
+    _hipcc(["-shared"] + sources + ["-o", output + ".tmp"], os.path.basename(output), verbose)
     os.replace(output + ".tmp", output)
     return output
+
+
+def _compile_library(verbose):
+    """Every translation unit of libfp6mi.so to an object (in parallel: the kernels of each format take most of the time),
+    then one link."""
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    objs = [os.path.join(OBJ_DIR, o) for _, o, _ in UNITS]
+
+    def one(unit):
+        src, obj, flags = unit
+        _hipcc(["-c", os.path.join(HERE, "csrc", src), "-o", os.path.join(OBJ_DIR, obj)] + flags, obj, verbose)
+    with ThreadPoolExecutor(max_workers=min(len(UNITS), os.cpu_count() or 1)) as pool:
+        list(pool.map(one, UNITS))
+    _hipcc(["-shared"] + objs + ["-o", OUTPUT + ".tmp"], "libfp6mi.so", verbose)
+    os.replace(OUTPUT + ".tmp", OUTPUT)
+    return OUTPUT
 
 
 def build_torch_extension(verbose=False):
@@ -63,7 +88,7 @@ def build(verbose=False):
     """Compiles every HIP/C++ source for gfx950 into libfp6mi.so and libfp6mi_probe.so, then the torch extension over the C
     ABI (always recompiles)."""
     _compile(PROBE_SOURCES, PROBE_OUTPUT, verbose)
-    lib = _compile(SOURCES, OUTPUT, verbose)
+    lib = _compile_library(verbose)
     build_torch_extension(verbose)
     return lib
 

@@ -1,8 +1,10 @@
-// gfx950 (MI355X) kernels of the FPx x FP16 linear layer, their launchers and the C ABI.
+// gfx950 (MI355X) kernels of the FPx x FP16 linear layer and their launchers, for ONE weight format per translation unit:
+// the build compiles this file once per format with -DFP6MI_FORMAT=<10*E+M> (32, 22, 23, 21), in parallel, and each object
+// exports one table of entry functions (fp6mi::FormatOps) that the C ABI in fp6mi_api.hip dispatches to.
 //
 // Roles taken over from the reference (usyd-fsalab/fp6_llm, paths relative to it):
 //   gemm_stream   <- QUANT_GEMM_Kernel        fp6_llm/csrc/include/kernel_matmul.cuh:29-191
-//   splitk_reduce <- SplitK_Reduction         fp6_llm/csrc/include/kernel_reduction.cuh:28-47
+//   splitk_reduce <- SplitK_Reduction         fp6_llm/csrc/include/kernel_reduction.cuh:28-47   (in fp6mi_api.hip)
 //   launchers     <- fpx_linear_kernel        fp6_llm/csrc/fp6_linear.cu:44-102
 // The design is not a translation: weights use the native layout described in fp6mi_host.cpp, go from HBM straight
 // to VGPRs with 128-bit non-temporal loads, FP6 codes are converted by the CDNA4 instruction
@@ -13,14 +15,17 @@
 // applied once to the FP32 sums instead of to every weight.
 #include <hip/hip_runtime.h>
 
-#include <mutex>
 #include <type_traits>
-#include <unordered_map>
-#include <vector>
 
 #include "fp6mi_internal.h"
 
+#ifndef FP6MI_FORMAT
+#error "compile with -DFP6MI_FORMAT=32, 22, 23 or 21 (10*E + M of the weight format)"
+#endif
+
 namespace {
+
+using fp6mi::LaunchCfg;
 
 typedef _Float16 half_t;
 typedef _Float16 v8h __attribute__((ext_vector_type(8)));
@@ -474,18 +479,6 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     }
 }
 
-// C[i] = fp16_rn(sum over splits, in split order, of ws[s][i]); four outputs per thread.
-__global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK)
-{
-    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= MN) return;
-    v4f sum = { 0.f, 0.f, 0.f, 0.f };
-    for (int s = 0; s < splitK; s++) sum += *reinterpret_cast<const v4f *>(ws + (size_t)s * MN + i);
-    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-    v4h o = { (half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3] };
-    *reinterpret_cast<v4h *>(C + i) = o;
-}
-
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
 template <int FM>
 __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, const uint8_t *__restrict__ W,
@@ -711,19 +704,7 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
     }
     store_native_lane<FM>(c, native + (size_t)blk * Fmt<FM>::block_bytes, lane);
 }
-
 // ------------------------------------------------------------------------------------------------ launch helpers
-
-inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
-
-// Calls fn with the format tag of a supported (E, M) as an integral constant.
-template <class Fn> inline int with_format(int E, int Mb, Fn &&fn)
-{
-    if (E == 3) return fn(std::integral_constant<int, 32>{});
-    if (Mb == 2) return fn(std::integral_constant<int, 22>{});
-    if (Mb == 3) return fn(std::integral_constant<int, 23>{});
-    return fn(std::integral_constant<int, 21>{});
-}
 
 template <int FM, int NT, int RT, int WAVES>
 int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
@@ -760,164 +741,7 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
                        ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
     return (int)hipGetLastError();
 }
-
 // kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
-struct LaunchCfg { int kind, nt, rt, wr, wk; };
-
-// Rule for batches above 16 where no measured neighbour exists: score the six tile shapes that exhaustive sweeps showed to
-// cover every case (64x32 with four K wavefronts; 128x32 with one or two; 128x64 with two; 256x64; 256x128) and take the
-// best.  The score is the product of
-//   * how full the chip is: workgroups / slots (one workgroup per CU, two for four-wavefront workgroups), divided by the
-//     number of rounds that takes when there are more workgroups than slots;
-//   * the share of the tile's columns that are real batch columns;
-//   * pipeline fill: chunks / (chunks + 2), a workgroup with few K chunks is mostly prologue and epilogue;
-//   * 1 / (1 + 32 * bytes through the CU's L1 per multiply-accumulate), which favours large tiles.
-// Against an exhaustive sweep (99 problems, all compiled shapes) the choice loses 0.6 % on average and 15 % at worst.
-struct TileShape { int nt, rt, wr, wk; };
-constexpr TileShape kRuleShapes[] = { { 2, 1, 4, 4 }, { 2, 2, 4, 1 }, { 2, 2, 4, 2 }, { 4, 2, 4, 2 }, { 4, 2, 8, 1 }, { 8, 2, 8, 1 } };
-
-inline double tile_score(size_t M, size_t N, size_t K, int splitK, const TileShape &t, int cus)
-{
-    const size_t TM = (size_t)t.wr * t.rt * 16, TN = (size_t)t.nt * 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
-    if (M % TM || (size_t)t.wk > per_split) return 0.0;
-    const size_t nblocks = (N + TN - 1) / TN;
-    const double wgs = (double)(M / TM) * nblocks * splitK, slots = (double)cus * (t.wr * t.wk <= 4 ? 2 : 1);
-    const double fill = wgs / slots, eff = fill >= 1.0 ? fill / std::ceil(fill) : fill;
-    const double cover = (double)N / (double)(nblocks * TN);
-    const double chunks = (double)per_split / t.wk, pipe = chunks / (chunks + 2.0);
-    const double traffic = (0.75 * TM + 2.0 * TN) / ((double)TM * TN);
-    return eff * cover * pipe / (1.0 + 32.0 * traffic);
-}
-
-// Estimated time in ns of the best shape for a given splitK: weight bytes at 6 TB/s divided by the score, plus, for a split, a
-// second launch (2 us) and the FP32 partial sums written and read back (8 bytes per output per split at 8 TB/s).
-inline double tile_estimate_ns(size_t M, size_t N, size_t K, int splitK, int cus, const TileShape **best_shape)
-{
-    double best = 0.0;
-    for (const TileShape &t : kRuleShapes) {
-        double sc = tile_score(M, N, K, splitK, t, cus);
-        if (sc > best) { best = sc; if (best_shape) *best_shape = &t; }
-    }
-    if (best <= 0.0) return 1e30;
-    double ns = (double)M * K * 0.75 / 6000.0 / best;
-    if (splitK > 1) ns += 2000.0 + (double)splitK * M * N * 8.0 / 8000.0;
-    return ns;
-}
-
-// ---- measured launch shapes (generated by `python -m fp6_llm_amd.tune`, MI355X, 256 CUs) ----
-struct TuneCfg { uint8_t kind, nt, rt, wr, wk; uint16_t t; };              // t in 0.02 us; kind 255 = not measured
-struct TuneEntry { uint8_t xb; uint16_t m256, k64, n; TuneCfg sk[4]; };    // sk[i]: best shape for splitK = 1 << i
-const TuneEntry kTune[] = {
-    { 0, 0, 0, 0, { { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 } } }, // keeps the array non-empty
-#include "fp6mi_tuning.inc"
-};
-
-inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (16u * c.rt * (c.kind == 1 ? c.wr : 1u)) == 0; }
-
-// Nearest measured problem: the batch is rounded UP to a measured batch of the same kernel family (a shape's cost steps at
-// column-tile boundaries), M and K go to the nearest measured value in ratio, at most a factor 1.5 away.
-struct TuneGroup { int xb; size_t n, begin, end; }; // entries [begin, end) of kTune share format and batch (the table is sorted by them)
-
-const std::vector<TuneGroup> &tune_groups()
-{
-    static const std::vector<TuneGroup> groups = [] {
-        std::vector<TuneGroup> g;
-        const size_t           count = sizeof(kTune) / sizeof(kTune[0]);
-        for (size_t i = 1; i < count; i++) {
-            if (g.empty() || g.back().xb != kTune[i].xb || g.back().n != kTune[i].n) g.push_back(TuneGroup{ kTune[i].xb, kTune[i].n, i, i });
-            g.back().end = i + 1;
-        }
-        return g;
-    }();
-    return groups;
-}
-
-const TuneEntry *tune_lookup(int xbits, size_t M, size_t N, size_t K)
-{
-    // a serving loop asks for the same few layer shapes at whatever batch size the scheduler formed: remember answers
-    struct Memo { int xb; size_t M, N, K; const TuneEntry *e; };
-    static thread_local Memo memo[256];
-    Memo &slot = memo[(M * 0x9E3779B97F4A7C15ull + N * 0xC2B2AE3D27D4EB4Full + K * 0x165667B19E3779F9ull + (size_t)xbits) >> 56];
-    if (slot.xb == xbits && slot.M == M && slot.N == N && slot.K == K) return slot.e;
-    const TuneGroup *group = nullptr, *widest = nullptr;
-    for (const TuneGroup &g : tune_groups()) {
-        if (g.xb != xbits || (g.n <= 16) != (N <= 16)) continue;
-        if (g.n >= N && (!group || g.n < group->n)) group = &g;
-        if (!widest || g.n > widest->n) widest = &g;
-    }
-    if (!group) group = widest; // batches beyond the largest measured one behave like it, only with more column blocks
-    const TuneEntry *best = nullptr;
-    float            best_d = 0.f;
-    if (group) {
-        const float lm = std::log2((float)M / 256.f), lk = std::log2((float)K / 64.f);
-        for (size_t i = group->begin; i < group->end; i++) {
-            const TuneEntry &e = kTune[i];
-            float dm = std::fabs(lm - std::log2((float)e.m256)), dk = std::fabs(lk - std::log2((float)e.k64));
-            if (dm > 0.585f || dk > 0.585f) continue;
-            if (!best || dm + dk < best_d) { best = &e; best_d = dm + dk; }
-        }
-    }
-    slot = Memo{ xbits, M, N, K, best };
-    return best;
-}
-
-// Launch shape for a given splitK.
-//  N <= 16: stream kernel.  Row tiles per wavefront (rt) reuse the activation registers, so rt grows with M; wavefronts
-//           per workgroup follow the K blocks of one split and the register budget (16 wavefronts leave 128 VGPRs each).
-//  N > 16:  tile kernel, 128 rows x 32 or 64 columns, with the K parallelism that splitK leaves open given to the
-//           wavefronts of the workgroup (at most what its LDS holds).
-inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, int cus)
-{
-    LaunchCfg c;
-    if (cus == 256 && (splitK == 1 || splitK == 2 || splitK == 4 || splitK == 8)) {
-        if (const TuneEntry *e = tune_lookup(xbits, M, N, K)) {
-            const TuneCfg &t = e->sk[splitK == 1 ? 0 : splitK == 2 ? 1 : splitK == 4 ? 2 : 3];
-            if (cfg_fits(t, M)) return LaunchCfg{ t.kind, t.nt, t.rt, t.wr, t.wk };
-        }
-    }
-    size_t    tiles = M / 16, units = (K + 255) / 256, per_split = (units + splitK - 1) / splitK;
-    if (N <= 16) {
-        c.kind = 0;
-        c.nt = 1;
-        c.wr = 1;
-        // Fitted to a sweep of every compiled shape over M in 2048..28672, K in 4096..28672, N in 1..16, both formats, on
-        // the MI355X.  What it encodes: about eight to eleven wavefronts per CU keep the memory system full; small
-        // workgroups (four wavefronts) balance better than large ones once there are several per CU; sharing the
-        // activation registers among row tiles (rt) pays in proportion to the batch, because every workgroup pulls the
-        // whole activation matrix through its CU's L1.
-        const double per_cu = (double)tiles * splitK / cus; // 16-row tiles per CU
-        if (N <= 4) {
-            if (per_cu < 1.5)        { c.rt = 1; c.wk = N <= 2 ? 16 : 8; }
-            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 8; }
-            else if (per_cu < 3.125) { c.rt = 1; c.wk = 4; }
-            else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
-            else                     { c.rt = 2; c.wk = 8; }
-        } else if (N <= 8) {
-            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
-            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 8; }
-            else if (per_cu < 3.125) { c.rt = 4; c.wk = 8; }
-            else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
-            else                     { c.rt = 4; c.wk = 4; }
-        } else {
-            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
-            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 4; }
-            else                     { c.rt = 4; c.wk = 4; }
-        }
-        while (c.rt > 1 && tiles % c.rt) c.rt /= 2;
-        const int cap = per_split > 8 ? 16 : per_split > 4 ? 8 : 4; // no more wavefronts than K blocks to hand out
-        if (c.wk > cap) c.wk = cap;
-        if (c.rt == 4 && c.wk == 16) c.wk = 8; // not compiled: 16 wavefronts leave too few registers for four row tiles
-        (void)xbits;
-        return c;
-    }
-    c.kind = 1;
-    const TileShape *t = nullptr;
-    tile_estimate_ns(M, N, K, splitK, cus, &t);
-    if (!t) t = &kRuleShapes[1]; // 128 x 32, one K wavefront: divides every legal M and needs a single K block
-    c.nt = t->nt, c.rt = t->rt, c.wr = t->wr, c.wk = t->wk;
-    return c;
-}
-
 template <int FM>
 int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
                size_t K, int splitK)
@@ -944,274 +768,66 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
     return FP6MI_ERR_SHAPE;
 }
 
+// ------------------------------------------------------------------------------------------------ entry functions of this format
+// (arguments are checked by the C ABI before it comes here)
 template <int FM>
-int linear_native(hipStream_t st, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
-                  int splitK, const LaunchCfg *forced)
+int op_gemm(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+            int splitK)
 {
-    LaunchCfg c = forced ? *forced : pick_cfg(Fmt<FM>::bits, M, N, K, splitK, 256);
-    if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
-    int rc = launch_cfg<FM>(c, st, W, sc, B, C, ws, M, N, K, splitK);
-    if (rc != 0) return rc;
-    if (splitK > 1) {
-        size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
-        hipLaunchKernelGGL(splitk_reduce, dim3((uint32_t)((MN / 4 + 255) / 256)), dim3(256), 0, st, static_cast<half_t *>(C), ws, MN,
-                           splitK);
-        rc = (int)hipGetLastError();
-    }
-    return rc;
+    return launch_cfg<FM>(c, static_cast<hipStream_t>(stream), W, sc, B, C, ws, M, N, K, splitK);
+}
+
+template <int FM> int op_relayout(void *stream, void *native, const void *ref, size_t M, size_t K)
+{
+    uint32_t units = (uint32_t)((K + 255) / 256);
+    size_t   blocks = (M / 16) * units;
+    hipLaunchKernelGGL(relayout_ref_to_native<FM>, dim3((uint32_t)((blocks + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint8_t *>(native), static_cast<const uint8_t *>(ref), (uint32_t)M, (uint32_t)K, units);
+    return (int)hipGetLastError();
+}
+
+template <int FM> int op_dequant(void *stream, void *out, const void *W, const void *sc, size_t M, size_t K)
+{
+    uint32_t units = (uint32_t)((K + 255) / 256);
+    size_t   blocks = (M / 16) * units;
+    hipLaunchKernelGGL(dequant_native<FM>, dim3((uint32_t)((blocks + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<half_t *>(out), static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
+    return (int)hipGetLastError();
+}
+
+// dtype: 0 = fp16, 1 = bf16, 2 = fp32
+template <int FM> int op_quantize(void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K)
+{
+    const uint32_t   units = (uint32_t)((K + 255) / 256);
+    const size_t     blocks = (M / 16) * units;
+    const dim3       grid_rows((uint32_t)((M + 3) / 4)), grid_blocks((uint32_t)((blocks + 3) / 4));
+    constexpr double max_value = Fmt<FM>::max_value;
+    hipStream_t      st = static_cast<hipStream_t>(stream);
+    uint8_t         *nat = static_cast<uint8_t *>(native);
+    half_t          *sc = static_cast<half_t *>(scales);
+    auto             run = [&](auto *typed) {
+        typedef std::remove_cv_t<std::remove_pointer_t<decltype(typed)>> T;
+        hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, typed, (uint32_t)M, (uint32_t)K, max_value);
+        hipLaunchKernelGGL((quant_to_native<FM, T>), grid_blocks, dim3(256), 0, st, nat, sc, typed, (uint32_t)M, (uint32_t)K, units, max_value);
+    };
+    if (dtype == 0)
+        run(static_cast<const half_t *>(weights));
+    else if (dtype == 1)
+        run(static_cast<const bf16_t *>(weights));
+    else
+        run(static_cast<const float *>(weights));
+    return (int)hipGetLastError();
 }
 
 } // namespace
 
-// ------------------------------------------------------------------------------------------------ C ABI
-
-extern "C" {
-
-const char *fp6mi_error_string(int code)
+namespace fp6mi {
+#define FP6MI_OPS_NAME_(f) format_ops_##f
+#define FP6MI_OPS_NAME(f) FP6MI_OPS_NAME_(f)
+const FormatOps &FP6MI_OPS_NAME(FP6MI_FORMAT)() // a host function, so that the table of host pointers stays out of the device code
 {
-    switch (code) {
-    case FP6MI_OK: return "success";
-    case FP6MI_ERR_FORMAT: return "unsupported (E,M): only FP6_e3m2 (3,2), FP5_e2m2 (2,2), FP6_e2m3 (2,3) and FP4_e2m1 (2,1)";
-    case FP6MI_ERR_SHAPE: return "unsupported shape: need M % 256 == 0 (64 for CPU packers, 16 for native packers), K % 64 == 0, N >= 1, distinct in/out";
-    case FP6MI_ERR_NULL: return "a required pointer is NULL";
-    case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
-    case FP6MI_ERR_SPLITK: return "splitK must be >= 1";
-    case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned";
-    default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fp6mi error";
-    }
+    static const FormatOps ops = { Fmt<FP6MI_FORMAT>::bits, &op_gemm<FP6MI_FORMAT>, &op_relayout<FP6MI_FORMAT>, &op_dequant<FP6MI_FORMAT>,
+                                   &op_quantize<FP6MI_FORMAT> };
+    return ops;
 }
-
-int fp6mi_version(void) { return 100; }
-
-int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
-int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }
-int fp6mi_dequant(int E, int Mb, void *out, const void *raw, size_t M, size_t K, const void *sc) { return fp6mi::dequant(E, Mb, out, raw, M, K, sc); }
-size_t fp6mi_native_bytes(int E, int Mb, size_t M, size_t K) { return fp6mi::native_bytes(E, Mb, M, K); }
-int fp6mi_prepack_native(int E, int Mb, void *native, const void *raw, size_t M, size_t K) { return fp6mi::prepack_native(E, Mb, native, raw, M, K); }
-int fp6mi_unpack_native(int E, int Mb, void *raw, const void *native, size_t M, size_t K) { return fp6mi::unpack_native(E, Mb, raw, native, M, K); }
-int fp6mi_relayout_ref_to_native(int E, int Mb, void *native, const void *ref, size_t M, size_t K)
-{
-    return fp6mi::relayout_ref_to_native(E, Mb, native, ref, M, K);
-}
-
-size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK) { return splitK > 1 ? (size_t)splitK * M * N * sizeof(float) : 0; }
-
-// Split-K choice.  Batches up to 16 (stream kernel): a cost model in microseconds on a part with `num_cus` compute
-// units -- workgroups run in rounds of one per CU, a workgroup streams its weights at what one CU sustains, the whole
-// chip cannot beat HBM, and a split costs a second launch plus writing and re-reading the FP32 partial sums; K is
-// already split inside the workgroup, so a split rarely pays.  Larger batches (tile kernel): as much of the wanted K
-// parallelism as keeps the FP32 partial-sum traffic (8 bytes per output per split) under half of the weight bytes.
-int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus)
-{
-    if (M == 0 || N == 0 || K == 0 || num_cus <= 0) return 1;
-    size_t units = (K + 255) / 256;
-    if (num_cus == 256) { // a measured neighbour knows better than any model: take its fastest split (3 % hysteresis towards fewer splits)
-        if (const TuneEntry *e = tune_lookup(6, M, N, K)) {
-            int      best_s = 0;
-            unsigned best_t = 0;
-            for (int i = 0; i < 4; i++) {
-                const TuneCfg &t = e->sk[i];
-                if (!cfg_fits(t, M) || (size_t)(1 << i) > units) continue;
-                if (best_s == 0 || (unsigned)t.t * 103u < best_t * 100u) { best_s = 1 << i; best_t = t.t; }
-            }
-            if (best_s) return best_s;
-        }
-    }
-    if (N > 16) {
-        int    best_s = 1;
-        double best_ns = 1e30;
-        for (int sp = 1; sp <= 8 && (size_t)sp <= units; sp *= 2) {
-            if (sp > 1 && (double)sp * 8.0 * (double)N > 0.75 * (double)K) break; // partial sums would outweigh the weights
-            double ns = tile_estimate_ns(M, N, K, sp, num_cus, nullptr);
-            if (ns < best_ns * 0.97) { best_ns = ns; best_s = sp; }
-        }
-        return best_s;
-    }
-    const double cu_gbps = 60.0, hbm_gbps = 6000.0, launch_us = 3.0;
-    size_t       wgs = M / 16 ? M / 16 : 1;
-    double       best = 1e30;
-    int          best_s = 1;
-    for (int s = 1; s <= 64 && (size_t)s <= units; s++) {
-        double per_wg_bytes = (double)((units + s - 1) / s) * 3072.0;
-        double rounds = std::ceil((double)(wgs * (size_t)s) / (double)num_cus);
-        double t_cu = rounds * per_wg_bytes / (cu_gbps * 1e3);
-        double t_hbm = (double)wgs * (double)units * 3072.0 / (hbm_gbps * 1e3);
-        double t = launch_us + (t_cu > t_hbm ? t_cu : t_hbm);
-        if (s > 1) t += launch_us + 2.0 * (double)s * (double)M * (double)N * 4.0 / (hbm_gbps * 1e3);
-        if (t < best * 0.97) { best = t; best_s = s; }
-    }
-    return best_s;
-}
-
-static int check_gemm_args(int E, int Mb, const void *W, const void *sc, const void *B, const void *C, size_t M, size_t N, size_t K,
-                           const float *ws, int splitK)
-{
-    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
-    if (!W || !sc || !B || !C) return FP6MI_ERR_NULL;
-    if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
-    if (M > 0x7fffffffu || N > 0x7fffffffu || K > 0x7fffffffu || (N + 15) / 16 > 65535) return FP6MI_ERR_SHAPE;
-    if (splitK < 1 || splitK > 65535) return FP6MI_ERR_SPLITK;
-    if (splitK > 1 && !ws) return FP6MI_ERR_WORKSPACE;
-    if (!aligned16(W) || !aligned16(B) || !aligned16(C) || (ws && !aligned16(ws))) return FP6MI_ERR_ALIGN;
-    return FP6MI_OK;
-}
-
-int fp6mi_linear_native(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
-                        float *ws, int splitK)
-{
-    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
-    if (rc != FP6MI_OK) return rc;
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    return with_format(E, Mb, [&](auto fm) { return linear_native<decltype(fm)::value>(st, W, sc, B, C, M, N, K, ws, splitK, nullptr); });
-}
-
-int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
-                            float *ws, int splitK, int kind, int n_tiles, int row_tiles, int row_waves, int k_waves)
-{
-    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
-    if (rc != FP6MI_OK) return rc;
-    LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    return with_format(E, Mb, [&](auto fm) { return linear_native<decltype(fm)::value>(st, W, sc, B, C, M, N, K, ws, splitK, &c); });
-}
-
-int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, int *shape)
-{
-    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
-    if (!shape) return FP6MI_ERR_NULL;
-    if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
-    if (splitK < 1) return FP6MI_ERR_SPLITK;
-    LaunchCfg c = pick_cfg(1 + E + Mb, M, N, K, splitK, 256);
-    shape[0] = c.kind, shape[1] = c.nt, shape[2] = c.rt, shape[3] = c.wr, shape[4] = c.wk;
-    return FP6MI_OK;
-}
-
-// ---- drop-in entry on REFERENCE-layout weights: native twins are made on first sight of a weight pointer and kept ----
-namespace {
-struct Twin { void *native; int E, Mb; size_t M, K; int device; };
-std::mutex                              g_twin_mutex;
-std::unordered_map<const void *, Twin>  g_twins;
-} // namespace
-
-int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
-                 float *ws, int splitK)
-{
-    int rc = check_gemm_args(E, Mb, W_ref, sc, B, C, M, N, K, ws, splitK);
-    if (rc != FP6MI_OK) return rc;
-    int device = 0;
-    if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return (int)e;
-    void *native = nullptr;
-    {
-        std::lock_guard<std::mutex> lock(g_twin_mutex);
-        auto it = g_twins.find(W_ref);
-        if (it != g_twins.end()) {
-            const Twin &t = it->second;
-            if (t.E == E && t.Mb == Mb && t.M == M && t.K == K && t.device == device) {
-                native = t.native;
-            } else { // the address now holds a different matrix
-                (void)hipFree(t.native);
-                g_twins.erase(it);
-            }
-        }
-        if (!native) {
-            size_t bytes = fp6mi::native_bytes(E, Mb, M, K);
-            if (hipError_t e = hipMalloc(&native, bytes); e != hipSuccess) return (int)e;
-            rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K); // same stream: ordered before the GEMM
-            if (rc != 0) {
-                (void)hipFree(native);
-                return rc;
-            }
-            g_twins[W_ref] = Twin{ native, E, Mb, M, K, device };
-        }
-    }
-    return fp6mi_linear_native(E, Mb, stream, native, sc, B, C, M, N, K, ws, splitK);
-}
-
-int fp6mi_twin_evict(const void *W_ref)
-{
-    std::lock_guard<std::mutex> lock(g_twin_mutex);
-    auto it = g_twins.find(W_ref);
-    if (it == g_twins.end()) return FP6MI_OK;
-    hipError_t e = hipFree(it->second.native); // hipFree waits for work that may still read the buffer
-    g_twins.erase(it);
-    return (int)e;
-}
-
-int fp6mi_twin_clear(void)
-{
-    std::lock_guard<std::mutex> lock(g_twin_mutex);
-    int rc = 0;
-    for (auto &kv : g_twins) {
-        hipError_t e = hipFree(kv.second.native);
-        if (e != hipSuccess) rc = (int)e;
-    }
-    g_twins.clear();
-    return rc;
-}
-
-int fp6mi_relayout_ref_to_native_gpu(int E, int Mb, void *stream, void *native, const void *ref, size_t M, size_t K)
-{
-    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
-    if (!native || !ref) return FP6MI_ERR_NULL;
-    if (M == 0 || M % 64 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu || native == ref) return FP6MI_ERR_SHAPE;
-    if (!aligned16(native) || !aligned16(ref)) return FP6MI_ERR_ALIGN;
-    uint32_t units = (uint32_t)((K + 255) / 256);
-    size_t   blocks = (M / 16) * units;
-    dim3     grid((uint32_t)((blocks + 3) / 4));
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    return with_format(E, Mb, [&](auto fm) {
-        hipLaunchKernelGGL(relayout_ref_to_native<decltype(fm)::value>, grid, dim3(256), 0, st, static_cast<uint8_t *>(native),
-                           static_cast<const uint8_t *>(ref), (uint32_t)M, (uint32_t)K, units);
-        return (int)hipGetLastError();
-    });
-}
-
-int fp6mi_dequant_native_gpu(int E, int Mb, void *stream, void *out, const void *W, const void *sc, size_t M, size_t K)
-{
-    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
-    if (!out || !W || !sc) return FP6MI_ERR_NULL;
-    if (M == 0 || M % 16 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu) return FP6MI_ERR_SHAPE;
-    if (!aligned16(out) || !aligned16(W)) return FP6MI_ERR_ALIGN;
-    uint32_t units = (uint32_t)((K + 255) / 256);
-    size_t   blocks = (M / 16) * units;
-    dim3     grid((uint32_t)((blocks + 3) / 4));
-    hipStream_t st = static_cast<hipStream_t>(stream);
-    return with_format(E, Mb, [&](auto fm) {
-        hipLaunchKernelGGL(dequant_native<decltype(fm)::value>, grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
-                           static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
-        return (int)hipGetLastError();
-    });
-}
-
-int fp6mi_quantize_native_gpu(int E, int Mb, void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K)
-{
-    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
-    if (!native || !scales || !weights) return FP6MI_ERR_NULL;
-    if (dtype < 0 || dtype > 2) return FP6MI_ERR_FORMAT;
-    if (M == 0 || M % 16 || K == 0 || K % 64 || M > 0x7fffffffu || K > 0x7fffffffu) return FP6MI_ERR_SHAPE;
-    if (!aligned16(native) || !aligned16(weights)) return FP6MI_ERR_ALIGN;
-    const uint32_t units = (uint32_t)((K + 255) / 256);
-    const size_t   blocks = (M / 16) * units;
-    const dim3     grid_rows((uint32_t)((M + 3) / 4)), grid_blocks((uint32_t)((blocks + 3) / 4));
-    hipStream_t    st = static_cast<hipStream_t>(stream);
-    uint8_t       *nat = static_cast<uint8_t *>(native);
-    half_t        *sc = static_cast<half_t *>(scales);
-    return with_format(E, Mb, [&](auto fm) {
-        constexpr int    FM = decltype(fm)::value;
-        constexpr double max_value = Fmt<FM>::max_value;
-        auto             run = [&](auto *typed) {
-            typedef std::remove_cv_t<std::remove_pointer_t<decltype(typed)>> T;
-            hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, typed, (uint32_t)M, (uint32_t)K, max_value);
-            hipLaunchKernelGGL((quant_to_native<FM, T>), grid_blocks, dim3(256), 0, st, nat, sc, typed, (uint32_t)M, (uint32_t)K, units, max_value);
-        };
-        if (dtype == 0)
-            run(static_cast<const half_t *>(weights));
-        else if (dtype == 1)
-            run(static_cast<const bf16_t *>(weights));
-        else
-            run(static_cast<const float *>(weights));
-        return (int)hipGetLastError();
-    });
-}
-
-} // extern "C"
+} // namespace fp6mi

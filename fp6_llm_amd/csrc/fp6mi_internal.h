@@ -13,6 +13,23 @@ namespace fp6mi {
 // FP6_e3m2 and FP5_e2m2 (the formats of the reference's entry points), FP6_e2m3 and FP4_e2m1 (through the same paths)
 inline bool supported(int E, int Mbits) { return (E == 3 && Mbits == 2) || (E == 2 && (Mbits == 1 || Mbits == 2 || Mbits == 3)); }
 
+// fp6mi_gemm.hip, compiled once per format: the entry functions of one weight format (stream = hipStream_t)
+// kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
+struct LaunchCfg { int kind, nt, rt, wr, wk; };
+struct FormatOps {
+    int bits;
+    int (*gemm)(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+                int splitK);
+    int (*relayout)(void *stream, void *native, const void *packed_ref, size_t M, size_t K);
+    int (*dequant)(void *stream, void *out_f16, const void *W, const void *sc, size_t M, size_t K);
+    int (*quantize)(void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K);
+};
+const FormatOps &format_ops_32(), &format_ops_22(), &format_ops_23(), &format_ops_21(); // named by 10*E + M
+inline const FormatOps *ops_for(int E, int Mbits)
+{
+    return E == 3 ? &format_ops_32() : Mbits == 2 ? &format_ops_22() : Mbits == 3 ? &format_ops_23() : &format_ops_21();
+}
+
 // fp6mi_host.cpp
 int    prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K);
 int    unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K);

@@ -29,7 +29,7 @@ TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 
 SPLITS = (1, 2, 4, 8)
 FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit width
 
-# every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip); the candidates above are the ones that
+# every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip, the same for every format); the candidates above are the ones that
 # ever came within 3 % of the best in exhaustive sweeps
 COMPILED_STREAM = [(0, nt, rt, 1, wk) for (nt, rt, wk) in
                    [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 4, 4), (1, 4, 8), (2, 1, 4), (2, 1, 8), (2, 2, 4),

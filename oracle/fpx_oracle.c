@@ -1,5 +1,5 @@
 /*
- * TEST INFRASTRUCTURE ONLY -- CPU restatement of the FPx (FP6_e3m2 / FP5_e2m2) linear-layer path of
+ * TEST INFRASTRUCTURE ONLY -- CPU restatement of the FPx (FP6_e3m2 / FP5_e2m2, also FP6_e2m3 / FP4_e2m1) linear-layer path of
  * usyd-fsalab/fp6_llm.  Nothing in the product links, loads or calls this file: only tests/,
  * __graft_entry__.smoke() and bench.py's cpu_baseline leg may use it, and only as the checker or as the
  * timed CPU baseline.
@@ -7,7 +7,7 @@
  * Plain scalar C, written to follow the reference's algorithm step by step (citations are paths relative to
  * the reference checkout, file:line).  It is deliberately slow and simple.
  *
- * What pins each function (see tests/test_oracle_*.py):
+ * What pins each function (see tests/test_oracle.py):
  *   orc_prepack      : byte-for-byte against the reference's own weight_prepacking.h compiled unmodified
  *                      (oracle/_ref), the all-ones known answers in tests/python/kernel_test_fpx.py:88-131,
  *                      an independent closed-form index formula, and bijection / in-place invariants.
@@ -16,6 +16,10 @@
  *                      the format constants of utils/weight_quant.h:22-25 (max 28, min subnormal 0.0625), and an
  *                      exhaustive check of every (code, fp16 scale sample) against the format definition evaluated in
  *                      exact rational arithmetic and rounded by Python's own IEEE binary16 packer.
+ *   e2m3, e2m1       : formats that only the reference's templates allow (its entry points reject them).  orc_prepack is
+ *                      pinned as above against the reference's prepacking template instantiated for those (E,M);
+ *                      orc_dequant for them is PARITY UNPINNED against reference output (none can be produced): it is
+ *                      pinned by the format definition in exact rationals and the OCP MX v1.0 constants only.
  *   orc_splitk_*     : closed forms (partition covers [0,K/64) exactly once, first K/64 % s splits one longer).
  *   orc_heuristic    : hand-computed known answers.
  *   orc_gemm         : the mathematical definition (fp32 accumulation of dequantized weights); checked against
