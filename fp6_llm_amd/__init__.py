@@ -170,9 +170,47 @@ def to_native(packed_tensor, EXPONENT=3, MANTISSA=2):
     return out
 
 
-def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC, IC):
+def group_exps_bytes(OC, IC):
+    n = _lib.lib().fp6mi_group_exps_bytes(OC, IC)
+    if n == 0:
+        raise ValueError("group exponents need OC % 16 == 0 and IC % 64 == 0")
+    return n
+
+
+def pack_group_exps(exps, OC, IC):
+    """Group exponents [OC, ceil(IC/128)] uint8 (factor 2^(b-127) on each group of 128 columns of a row; CPU tensor) -> the
+    1-D uint8 tensor in the order the kernels read."""
+    if exps.dtype != torch.uint8 or exps.dim() != 2 or exps.shape != (OC, (IC + 127) // 128) or exps.device.type != "cpu":
+        raise ValueError("exps must be a CPU uint8 tensor [OC, ceil(IC/128)]")
+    out = torch.empty(group_exps_bytes(OC, IC), dtype=torch.uint8)
+    _lib.check(_lib.lib().fp6mi_pack_group_exps(out.data_ptr(), exps.contiguous().data_ptr(), OC, IC), "fp6mi_pack_group_exps")
+    return out
+
+
+def weight_dequant_grouped_cpu(EXPONENT, MANTISSA, fpx_tensor, fp16_scale, exps):
+    """weight_dequant_eXmY_cpu with group exponents: fp16_rn(value * 2^(b-127) * scale[row]); exps [OC, ceil(IC/128)] uint8."""
+    OC, IC = _weight_shape(fpx_tensor, EXPONENT, MANTISSA, "fpx_tensor")
+    src = _cpu_contig(fpx_tensor, "fpx_tensor")
+    if fp16_scale.dtype != torch.float16 or fp16_scale.numel() != OC:
+        raise ValueError("fp16_scale must be float16 [OC]")
+    if exps.dtype != torch.uint8 or exps.shape != (OC, (IC + 127) // 128):
+        raise ValueError("exps must be uint8 [OC, ceil(IC/128)]")
+    out = torch.empty((OC, IC), dtype=torch.float16)
+    _lib.check(_lib.lib().fp6mi_dequant_grouped(EXPONENT, MANTISSA, out.data_ptr(), src.data_ptr(), OC, IC,
+                                                _cpu_contig(fp16_scale, "fp16_scale").data_ptr(), _cpu_contig(exps, "exps").data_ptr()),
+               "fp6mi_dequant_grouped")
+    return out
+
+
+def _check_group_exps(group_exps, OC, IC, dev):
+    if group_exps.dtype != torch.uint8 or group_exps.device != dev or not group_exps.is_contiguous() or \
+            group_exps.numel() != (OC // 16) * ((IC + 255) // 256) * 32:
+        raise ValueError("group_exps must be the contiguous uint8 tensor of pack_group_exps(exps, OC, IC) on the weights' GPU")
+
+
+def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC, IC, group_exps=None):
     """Native-layout weights on the GPU -> fp16 [OC, IC] with the GEMM's own in-register conversion (bit-exact to
-    weight_dequant_eXmY_cpu of the same weights)."""
+    weight_dequant_eXmY_cpu of the same weights; with group_exps, to weight_dequant_grouped_cpu)."""
     _bits(EXPONENT, MANTISSA)
     if native_weight.device.type != "cuda" or fp16_scale.device != native_weight.device:
         raise ValueError("native_weight and fp16_scale must be on the same GPU")
@@ -181,8 +219,14 @@ def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC
     out = torch.empty((OC, IC), dtype=torch.float16, device=native_weight.device)
     with torch.cuda.device(native_weight.device):
         stream = torch.cuda.current_stream().cuda_stream
-        _lib.check(_lib.lib().fp6mi_dequant_native_gpu(EXPONENT, MANTISSA, stream, out.data_ptr(), native_weight.data_ptr(),
-                                                       fp16_scale.contiguous().data_ptr(), OC, IC), "fp6mi_dequant_native_gpu")
+        if group_exps is None:
+            _lib.check(_lib.lib().fp6mi_dequant_native_gpu(EXPONENT, MANTISSA, stream, out.data_ptr(), native_weight.data_ptr(),
+                                                           fp16_scale.contiguous().data_ptr(), OC, IC), "fp6mi_dequant_native_gpu")
+        else:
+            _check_group_exps(group_exps, OC, IC, native_weight.device)
+            _lib.check(_lib.lib().fp6mi_dequant_native_grouped_gpu(EXPONENT, MANTISSA, stream, out.data_ptr(), native_weight.data_ptr(),
+                                                                   fp16_scale.contiguous().data_ptr(), group_exps.data_ptr(), OC, IC),
+                       "fp6mi_dequant_native_grouped_gpu")
     return out
 
 
@@ -235,10 +279,11 @@ def _workspace(device, stream, nbytes):
 _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)   # the current stream's handle without building a Stream object
 
 
-def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, splitK=1, out=None, workspace=None):
-    """out[B, OC] = in_feats[B, IC] @ dequant(W)^T with W in the native layout.  Enqueued on the current stream."""
+def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, splitK=1, out=None, workspace=None, group_exps=None):
+    """out[B, OC] = in_feats[B, IC] @ dequant(W)^T with W in the native layout.  Enqueued on the current stream.
+    group_exps: the tensor of pack_group_exps on the same GPU for weights with per-group exponents, else None."""
     if _ext is not None:
-        return _ext.linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, int(splitK), out, workspace)
+        return _ext.linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, OC, int(splitK), out, workspace, group_exps)
     _bits(EXPONENT, MANTISSA)
     if in_feats.dtype != torch.float16 or in_feats.dim() != 2:
         raise ValueError("in_feats must be a 2-D float16 tensor [B, IC]")
@@ -280,8 +325,13 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
             elif workspace.dtype != torch.float32 or workspace.numel() * 4 < need or workspace.device != dev:
                 raise ValueError("workspace must be a float32 GPU tensor with at least splitK*B*OC elements")
             ws_ptr = workspace.data_ptr()
-        rc = L.fp6mi_linear_native(EXPONENT, MANTISSA, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(),
-                                   out.data_ptr(), OC, B, IC, ws_ptr, splitK)
+        if group_exps is None:
+            rc = L.fp6mi_linear_native(EXPONENT, MANTISSA, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(),
+                                       out.data_ptr(), OC, B, IC, ws_ptr, splitK)
+        else:
+            _check_group_exps(group_exps, OC, IC, dev)
+            rc = L.fp6mi_linear_native_grouped(EXPONENT, MANTISSA, stream, native_weight.data_ptr(), sc.data_ptr(), group_exps.data_ptr(),
+                                               x.data_ptr(), out.data_ptr(), OC, B, IC, ws_ptr, splitK)
     finally:
         if switch:
             torch.cuda.set_device(prev)

@@ -109,18 +109,38 @@ template <int FM> __device__ __forceinline__ v6u field_string(const WFrag<FM> &f
         return fp4_expand(h == 0 ? f.a : f.b);
 }
 
-template <int FM> __device__ __forceinline__ v32h fields_to_halfs(v6u src)
+// The conversion instruction multiplies its 32 values by the power of two in the exponent field of `scale` at no cost.
+template <int FM> __device__ __forceinline__ v32h fields_to_halfs(v6u src, float scale)
 {
     if constexpr (Fmt<FM>::hw_e3m2)
-        return __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, 1.0f);
+        return __builtin_amdgcn_cvt_scalef32_pk32_f16_bf6(src, scale);
     else
-        return __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(src, 1.0f);
+        return __builtin_amdgcn_cvt_scalef32_pk32_f16_fp6(src, scale);
 }
 
-template <int FM> __device__ __forceinline__ void convert(const WFrag<FM> &f, AOps<FM> &o)
+// Group exponents: one byte b per (row, 128 columns), meaning the factor 2^(b-127) on those weights (the E8M0 scale type of
+// the OCP MX formats).  A lane's 32-code string is exactly its row's share of one 128-column group, so the factor rides on
+// the conversion instruction.  Native layout of the bytes: [row tile][K block][row in tile][half of the block], 32 bytes per
+// block; `g` below is the lane's pair of bytes (half 0 in the low byte).  GS = false: no group exponents, factor 1.
+template <bool GS> __device__ __forceinline__ float group_factor(uint32_t g, int h)
 {
-    v32h h0 = fields_to_halfs<FM>(field_string<FM>(f, 0));
-    v32h h1 = fields_to_halfs<FM>(field_string<FM>(f, 1));
+    if constexpr (GS)
+        return __builtin_bit_cast(float, (h == 0 ? (g & 0xffu) : (g >> 8)) << 23);
+    else
+        return 1.0f;
+}
+template <bool GS> __device__ __forceinline__ uint32_t load_group_exps(const uint8_t *gexp_block, int lane)
+{
+    if constexpr (GS)
+        return *reinterpret_cast<const uint16_t *>(gexp_block + 2 * (lane & 15));
+    else
+        return 0;
+}
+
+template <int FM, bool GS> __device__ __forceinline__ void convert(const WFrag<FM> &f, AOps<FM> &o, uint32_t g)
+{
+    v32h h0 = fields_to_halfs<FM>(field_string<FM>(f, 0), group_factor<GS>(g, 0));
+    v32h h1 = fields_to_halfs<FM>(field_string<FM>(f, 1), group_factor<GS>(g, 1));
 #pragma unroll
     for (int i = 0; i < 4; i++) {
         o.s[i]     = slice8(h0, i);
@@ -155,15 +175,20 @@ template <int NT> __device__ __forceinline__ void load_x_paired(v8h (&x)[8][NT],
 
 template <int FM, int NT, int RT> struct Stage {
     WFrag<FM> w[RT];
+    uint32_t  g[RT]; // group exponents of the block (unused without them)
     v8h       x[8][NT];
 };
 
-template <int FM, int NT, int RT>
-__device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, uint32_t u, int lane,
-                                           const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack, const half_t *xrow_packed)
+template <int FM, bool GS, int NT, int RT>
+__device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, const uint8_t *ggroup, uint32_t units,
+                                           uint32_t u, int lane, const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack,
+                                           const half_t *xrow_packed)
 {
 #pragma unroll
-    for (int r = 0; r < RT; r++) st.w[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
+    for (int r = 0; r < RT; r++) {
+        st.w[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
+        st.g[r] = load_group_exps<GS>(ggroup + ((size_t)r * units + u) * 32, lane);
+    }
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
     // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
@@ -187,13 +212,13 @@ __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t 
     __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
 }
 
-template <int FM, int NT, int RT>
+template <int FM, bool GS, int NT, int RT>
 __device__ __forceinline__ void consume_stage(const Stage<FM, NT, RT> &st, v4f (&acc)[RT][NT])
 {
 #pragma unroll
     for (int r = 0; r < RT; r++) {
         AOps<FM> a;
-        convert(st.w[r], a);
+        convert<FM, GS>(st.w[r], a, st.g[r]);
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
@@ -201,9 +226,9 @@ __device__ __forceinline__ void consume_stage(const Stage<FM, NT, RT> &st, v4f (
     }
 }
 
-template <int FM, int NT, int RT, int WAVES>
+template <int FM, bool GS, int NT, int RT, int WAVES>
 __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
-                                                            const half_t *__restrict__ X, half_t *__restrict__ C,
+                                                            const uint8_t *__restrict__ gexp, const half_t *__restrict__ X, half_t *__restrict__ C,
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
                                                             uint32_t units, uint32_t splitK)
 {
@@ -219,6 +244,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 
     const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
+    const uint8_t *ggroup = GS ? gexp + (size_t)R0 * units * 32 : nullptr;
 
     v4f acc[RT][NT];
 #pragma unroll
@@ -253,8 +279,8 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     // busy while this one converts, and a second stage in registers measured slower at every size.
     for (uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES); u < u1; u += WAVES) {
         Stage<FM, NT, RT> cur;
-        load_stage<FM, NT, RT>(cur, wgroup, tile_stride, u, lane, xrow, q, K, xpack, xrow_packed);
-        consume_stage<FM, NT, RT>(cur, acc);
+        load_stage<FM, GS, NT, RT>(cur, wgroup, tile_stride, ggroup, units, u, lane, xrow, q, K, xpack, xrow_packed);
+        consume_stage<FM, GS, NT, RT>(cur, acc);
     }
 
     // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
@@ -286,9 +312,9 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 }
 
 // A operands of MFMA steps 4h..4h+3 (half of a K block) of one lane.
-template <int FM> __device__ __forceinline__ void convert_half(const WFrag<FM> &f, int h, v8h (&o)[4])
+template <int FM, bool GS> __device__ __forceinline__ void convert_half(const WFrag<FM> &f, int h, v8h (&o)[4], uint32_t g)
 {
-    v32h v = fields_to_halfs<FM>(field_string<FM>(f, h));
+    v32h v = fields_to_halfs<FM>(field_string<FM>(f, h), group_factor<GS>(g, h));
 #pragma unroll
     for (int i = 0; i < 4; i++) o[i] = slice8(v, i);
 }
@@ -307,9 +333,9 @@ template <int FM> __device__ __forceinline__ void convert_half(const WFrag<FM> &
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kXsRowBytes = 544;
 
-template <int FM, int NT, int RT, int WR, int WK>
+template <int FM, bool GS, int NT, int RT, int WR, int WK>
 __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
-                                                           const half_t *__restrict__ X, half_t *__restrict__ C,
+                                                           const uint8_t *__restrict__ gexp, const half_t *__restrict__ X, half_t *__restrict__ C,
                                                            float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
                                                            uint32_t units, uint32_t splitK, uint32_t nblocks)
 {
@@ -335,6 +361,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 
     const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
+    const uint8_t *ggroup = GS ? gexp + (size_t)R0 * units * 32 : nullptr;
 
     v4f acc[RT][NT];
 #pragma unroll
@@ -343,6 +370,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
 
     WFrag<FM> wcur[RT], wnxt[RT];
+    uint32_t  gcur[RT], gnxt[RT]; // group exponents travel with the weights (unused without them)
     v4u       xr[kPerThread];
 
     // row scales of this lane's outputs (rows 4q..4q+3 of each of its row tiles), fetched before the main loop so that no
@@ -352,11 +380,14 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
     for (int r = 0; r < RT; r++) sc4[r] = *reinterpret_cast<const v4h *>(scales + (R0 + r) * 16 + 4 * q);
 
-    auto load_w = [&](WFrag<FM>(&dst)[RT], uint32_t c0) {
+    auto load_w = [&](WFrag<FM>(&dst)[RT], uint32_t(&gdst)[RT], uint32_t c0) {
         const uint32_t u = c0 + wk;
         if (u < u1) {
 #pragma unroll
-            for (int r = 0; r < RT; r++) dst[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
+            for (int r = 0; r < RT; r++) {
+                dst[r]  = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
+                gdst[r] = load_group_exps<GS>(ggroup + ((size_t)r * units + u) * 32, lane);
+            }
         }
     };
     // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
@@ -396,7 +427,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 
     if (u0 < u1) {
         load_x(u0);
-        load_w(wcur, u0);
+        load_w(wcur, gcur, u0);
         store_x(0);
         __syncthreads();
         int buf = 0;
@@ -404,16 +435,16 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
             const bool more = c0 + WK < u1;
             if (more) {
                 load_x(c0 + WK);
-                load_w(wnxt, c0 + WK);
+                load_w(wnxt, gnxt, c0 + WK);
             }
             if (c0 + wk < u1) {
                 const uint8_t *xs = lds + buf * kBufBytes + (wk * TN + col) * kXsRowBytes + q * 16;
                 v8h            a0[RT][4], a1[RT][4];
 #pragma unroll
-                for (int r = 0; r < RT; r++) convert_half(wcur[r], 0, a0[r]);
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 0, a0[r], gcur[r]);
                 // second half converted ahead of the first half's MFMAs: the VALU work then runs under the matrix pipe
 #pragma unroll
-                for (int r = 0; r < RT; r++) convert_half(wcur[r], 1, a1[r]);
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 1, a1[r], gcur[r]);
 #pragma unroll
                 for (int h = 0; h < 2; h++) {
 #pragma unroll
@@ -432,7 +463,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
             if (more) {
                 store_x(buf ^ 1); // that buffer was last read before the barrier that ended the previous iteration
 #pragma unroll
-                for (int r = 0; r < RT; r++) wcur[r] = wnxt[r];
+                for (int r = 0; r < RT; r++) wcur[r] = wnxt[r], gcur[r] = gnxt[r];
             }
             __syncthreads();
         }
@@ -480,9 +511,9 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 }
 
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
-template <int FM>
-__global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, const uint8_t *__restrict__ W,
-                                                     const half_t *__restrict__ scales, uint32_t M, uint32_t K, uint32_t units)
+template <int FM, bool GS>
+__global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
+                                                     const uint8_t *__restrict__ gexp, uint32_t M, uint32_t K, uint32_t units)
 {
     const int      lane = threadIdx.x & 63;
     const uint32_t blk = blockIdx.x * 4 + (threadIdx.x >> 6);
@@ -491,7 +522,7 @@ __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, 
     const int      m = lane & 15, q = lane >> 4;
     WFrag<FM>      wf = load_wfrag<FM>(W + (size_t)blk * Fmt<FM>::block_bytes, lane);
     AOps<FM>       a;
-    convert(wf, a);
+    convert<FM, GS>(wf, a, load_group_exps<GS>(gexp + (size_t)blk * 32, lane));
     const half_t sc = scales[R * 16 + m], post = (half_t)Fmt<FM>::post_scale;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
@@ -706,20 +737,21 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
 }
 // ------------------------------------------------------------------------------------------------ launch helpers
 
-template <int FM, int NT, int RT, int WAVES>
-int launch_stream(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+template <int FM, bool GS, int NT, int RT, int WAVES>
+int launch_stream(hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
                   int splitK)
 {
     uint32_t units = (uint32_t)((K + 255) / 256);
     dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    hipLaunchKernelGGL((gemm_stream<FM, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
-                       static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M,
-                       (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
+    hipLaunchKernelGGL((gemm_stream<FM, GS, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
+                       static_cast<const half_t *>(sc), static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws,
+                       (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
     return (int)hipGetLastError();
 }
 
-template <int FM, int NT, int RT, int WR, int WK>
-int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K, int splitK)
+template <int FM, bool GS, int NT, int RT, int WR, int WK>
+int launch_tile(hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+                int splitK)
 {
     constexpr int TN = NT * 16, TM = WR * RT * 16;
     constexpr size_t x_bytes = 2 * (size_t)WK * TN * kXsRowBytes, red_bytes = WK > 1 ? (size_t)WK * WR * RT * NT * 1024 : 0;
@@ -728,7 +760,7 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
     if (M % TM) return FP6MI_ERR_SHAPE;
     static bool attr_set = false; // idempotent, so a race between host threads is harmless
     if (!attr_set && lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, NT, RT, WR, WK>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, GS, NT, RT, WR, WK>),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if (e != hipSuccess) return (int)e;
         attr_set = true;
@@ -736,19 +768,19 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *B, vo
     uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
     size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
     if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
-    hipLaunchKernelGGL((gemm_tile<FM, NT, RT, WR, WK>), dim3((uint32_t)wgs), dim3(WR * WK * kWave), lds_bytes, st,
-                       static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), static_cast<const half_t *>(B), static_cast<half_t *>(C),
-                       ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
+    hipLaunchKernelGGL((gemm_tile<FM, GS, NT, RT, WR, WK>), dim3((uint32_t)wgs), dim3(WR * WK * kWave), lds_bytes, st,
+                       static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B),
+                       static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
     return (int)hipGetLastError();
 }
 // kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
-template <int FM>
-int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N,
-               size_t K, int splitK)
+template <int FM, bool GS>
+int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M,
+               size_t N, size_t K, int splitK)
 {
     if (c.kind == 0) {
 #define FP6MI_CASE(NT, RT, WV) \
-    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<FM, NT, RT, WV>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<FM, GS, NT, RT, WV>(st, W, sc, gexp, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
         FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
@@ -759,7 +791,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
 #undef FP6MI_CASE
     } else if (c.kind == 1) {
 #define FP6MI_CASE(NT, RT, WR, WK) \
-    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<FM, NT, RT, WR, WK>(st, W, sc, B, C, ws, M, N, K, splitK);
+    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == WK) return launch_tile<FM, GS, NT, RT, WR, WK>(st, W, sc, gexp, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
         FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
         FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1) FP6MI_CASE(4, 1, 4, 2) FP6MI_CASE(2, 1, 2, 4)
@@ -770,11 +802,13 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
 
 // ------------------------------------------------------------------------------------------------ entry functions of this format
 // (arguments are checked by the C ABI before it comes here)
+// gexp: group exponents in their native layout, or null for none
 template <int FM>
-int op_gemm(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
-            int splitK)
+int op_gemm(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M,
+            size_t N, size_t K, int splitK)
 {
-    return launch_cfg<FM>(c, static_cast<hipStream_t>(stream), W, sc, B, C, ws, M, N, K, splitK);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return gexp ? launch_cfg<FM, true>(c, st, W, sc, gexp, B, C, ws, M, N, K, splitK) : launch_cfg<FM, false>(c, st, W, sc, nullptr, B, C, ws, M, N, K, splitK);
 }
 
 template <int FM> int op_relayout(void *stream, void *native, const void *ref, size_t M, size_t K)
@@ -786,12 +820,18 @@ template <int FM> int op_relayout(void *stream, void *native, const void *ref, s
     return (int)hipGetLastError();
 }
 
-template <int FM> int op_dequant(void *stream, void *out, const void *W, const void *sc, size_t M, size_t K)
+template <int FM> int op_dequant(void *stream, void *out, const void *W, const void *sc, const void *gexp, size_t M, size_t K)
 {
-    uint32_t units = (uint32_t)((K + 255) / 256);
-    size_t   blocks = (M / 16) * units;
-    hipLaunchKernelGGL(dequant_native<FM>, dim3((uint32_t)((blocks + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<half_t *>(out), static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), (uint32_t)M, (uint32_t)K, units);
+    uint32_t    units = (uint32_t)((K + 255) / 256);
+    size_t      blocks = (M / 16) * units;
+    dim3        grid((uint32_t)((blocks + 3) / 4));
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (gexp)
+        hipLaunchKernelGGL((dequant_native<FM, true>), grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
+                           static_cast<const half_t *>(sc), static_cast<const uint8_t *>(gexp), (uint32_t)M, (uint32_t)K, units);
+    else
+        hipLaunchKernelGGL((dequant_native<FM, false>), grid, dim3(256), 0, st, static_cast<half_t *>(out), static_cast<const uint8_t *>(W),
+                           static_cast<const half_t *>(sc), static_cast<const uint8_t *>(nullptr), (uint32_t)M, (uint32_t)K, units);
     return (int)hipGetLastError();
 }
 

@@ -202,13 +202,15 @@ int unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K)
 // value(code) = (-1)^s 2^(e-b) (1+m/2^M), e = 0: (-1)^s 2^(1-b) m/2^M, b = 2^(E-1)-1; every exponent is an ordinary value.
 // out = fp16_rn(value * float(scale)): the product of an at most 4-bit and an 11-bit significand is exact in FP32, so there is
 // one rounding, which is what utils/weight_dequant.h:30-43 of the reference computes.
-int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16)
+// exps (may be null): one byte b per (row, 128 columns), row-major [M][ceil(K/128)], the factor 2^(b-127) on those weights;
+// then out = fp16_rn(value * 2^(b-127) * float(scale)), still one rounding (the power of two is exact in double).
+static int dequant_any(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16, const uint8_t *exps)
 {
     if (!supported(E, Mb)) return FP6MI_ERR_FORMAT;
     if (!out_f16 || !raw || !scales_f16) return FP6MI_ERR_NULL;
     if (M == 0 || K == 0 || K % 8) return FP6MI_ERR_SHAPE;
     int    x = 1 + E + Mb, ncodes = 1 << x;
-    size_t row_bytes = K * x / 8;
+    size_t row_bytes = K * x / 8, groups = (K + 127) / 128;
     float  value[64];
     for (int c = 0; c < ncodes; c++) {
         int   s = c >> (x - 1), e = (c >> Mb) & ((1 << E) - 1), m = c & ((1 << Mb) - 1), b = (1 << (E - 1)) - 1;
@@ -223,12 +225,50 @@ int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, c
         for (size_t r = blk * 16; r < std::min(M, blk * 16 + 16); r++) {
             _Float16 table[64];
             float    s = (float)sc[r];
-            for (int c = 0; c < ncodes; c++) table[c] = (_Float16)(value[c] * s); // float -> half is round-to-nearest-even
             read_codes(src + r * row_bytes, x, 0, K, codes.data());
             _Float16 *o = dst + r * K;
-            for (size_t c = 0; c < K; c++) o[c] = table[codes[c]];
+            for (size_t g = 0; g < (exps ? groups : 1); g++) {
+                // value * 2^k * scale has at most 4 + 11 significant bits: exact in double for every k, and exact in float
+                // wherever fp16 can tell the result from zero or infinity; so the float -> half step is the one rounding
+                double f = exps ? std::ldexp(1.0, (int)exps[r * groups + g] - 127) : 1.0;
+                for (int c = 0; c < ncodes; c++) table[c] = (_Float16)(float)((double)value[c] * f * (double)s);
+                size_t c0 = exps ? g * 128 : 0, c1 = exps ? std::min(K, c0 + 128) : K;
+                for (size_t c = c0; c < c1; c++) o[c] = table[codes[c]];
+            }
         }
     });
+    return FP6MI_OK;
+}
+
+int dequant(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16)
+{
+    return dequant_any(E, Mb, out_f16, raw, M, K, scales_f16, nullptr);
+}
+
+int dequant_grouped(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16, const void *exps)
+{
+    if (!exps) return FP6MI_ERR_NULL;
+    return dequant_any(E, Mb, out_f16, raw, M, K, scales_f16, static_cast<const uint8_t *>(exps));
+}
+
+// Group exponents in the order the kernels read them: [row tile][K block][row in tile][half of the block], 32 bytes per
+// 16x256 block; halves beyond K hold 127 (factor 1; the weights there are zero codes anyway).
+size_t group_exps_bytes(size_t M, size_t K) { return (M % 16 || K % 64) ? 0 : (M / 16) * ((K + 255) / 256) * 32; }
+
+int pack_group_exps(void *native_exps, const void *exps, size_t M, size_t K)
+{
+    if (!native_exps || !exps) return FP6MI_ERR_NULL;
+    if (M == 0 || K == 0 || M % 16 || K % 64 || native_exps == exps) return FP6MI_ERR_SHAPE;
+    const size_t   units = (K + 255) / 256, groups = (K + 127) / 128;
+    const uint8_t *src = static_cast<const uint8_t *>(exps);
+    uint8_t       *dst = static_cast<uint8_t *>(native_exps);
+    for (size_t R = 0; R < M / 16; R++)
+        for (size_t U = 0; U < units; U++)
+            for (size_t m = 0; m < 16; m++)
+                for (size_t h = 0; h < 2; h++) {
+                    size_t g = 2 * U + h;
+                    dst[((R * units + U) * 16 + m) * 2 + h] = g < groups ? src[(R * 16 + m) * groups + g] : (uint8_t)127;
+                }
     return FP6MI_OK;
 }
 

@@ -18,10 +18,11 @@ inline bool supported(int E, int Mbits) { return (E == 3 && Mbits == 2) || (E ==
 struct LaunchCfg { int kind, nt, rt, wr, wk; };
 struct FormatOps {
     int bits;
-    int (*gemm)(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
-                int splitK);
+    // gexp: group exponents in their native layout (one byte per row and 128 columns), or null
+    int (*gemm)(const LaunchCfg &c, void *stream, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M,
+                size_t N, size_t K, int splitK);
     int (*relayout)(void *stream, void *native, const void *packed_ref, size_t M, size_t K);
-    int (*dequant)(void *stream, void *out_f16, const void *W, const void *sc, size_t M, size_t K);
+    int (*dequant)(void *stream, void *out_f16, const void *W, const void *sc, const void *gexp, size_t M, size_t K);
     int (*quantize)(void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K);
 };
 const FormatOps &format_ops_32(), &format_ops_22(), &format_ops_23(), &format_ops_21(); // named by 10*E + M
@@ -39,6 +40,9 @@ size_t native_bytes(int E, int Mb, size_t M, size_t K);
 int    prepack_native(int E, int Mb, void *native, const void *raw, size_t M, size_t K);
 int    unpack_native(int E, int Mb, void *raw, const void *native, size_t M, size_t K);
 int    relayout_ref_to_native(int E, int Mb, void *native, const void *packed_ref, size_t M, size_t K);
+size_t group_exps_bytes(size_t M, size_t K);
+int    pack_group_exps(void *native_exps, const void *exps, size_t M, size_t K);
+int    dequant_grouped(int E, int Mb, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16, const void *exps);
 
 } // namespace fp6mi
 #endif

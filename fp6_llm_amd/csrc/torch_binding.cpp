@@ -37,7 +37,8 @@ at::Tensor workspace_for(const at::Device &dev, void *stream, int64_t floats)
 
 // out[B, OC] = in_feats[B, IC] @ dequant(W)^T with W in the native layout, enqueued on the current stream of in_feats' device.
 at::Tensor linear_forward_native(int64_t E, int64_t Mb, const at::Tensor &in_feats, const at::Tensor &native_weight, const at::Tensor &scales,
-                                 int64_t OC, int64_t splitK, const c10::optional<at::Tensor> &out_opt, const c10::optional<at::Tensor> &ws_opt)
+                                 int64_t OC, int64_t splitK, const c10::optional<at::Tensor> &out_opt, const c10::optional<at::Tensor> &ws_opt,
+                                 const c10::optional<at::Tensor> &gexp_opt)
 {
     const bool known = (E == 3 && Mb == 2) || (E == 2 && Mb >= 1 && Mb <= 3);
     if (!known) bad("unsupported format: EXPONENT=" + std::to_string(E) + ", MANTISSA=" + std::to_string(Mb) + " (only e3m2, e2m2, e2m3 and e2m1)");
@@ -76,8 +77,17 @@ at::Tensor linear_forward_native(int64_t E, int64_t Mb, const at::Tensor &in_fea
         }
         ws_ptr = ws.data_ptr<float>();
     }
-    int rc = fp6mi_linear_native((int)E, (int)Mb, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(), out.data_ptr(), (size_t)OC, (size_t)B,
+    int rc;
+    if (gexp_opt.has_value()) { // per-group exponents in the kernels' own order (fp6mi_pack_group_exps)
+        const at::Tensor &g = *gexp_opt;
+        if (g.scalar_type() != at::kByte || g.device() != dev || !g.is_contiguous() || g.numel() != (int64_t)fp6mi_group_exps_bytes((size_t)OC, (size_t)IC))
+            bad("group_exps must be the contiguous uint8 tensor of pack_group_exps(exps, OC, IC) on the weights' GPU");
+        rc = fp6mi_linear_native_grouped((int)E, (int)Mb, stream, native_weight.data_ptr(), sc.data_ptr(), g.data_ptr(), x.data_ptr(), out.data_ptr(),
+                                         (size_t)OC, (size_t)B, (size_t)IC, ws_ptr, (int)splitK);
+    } else {
+        rc = fp6mi_linear_native((int)E, (int)Mb, stream, native_weight.data_ptr(), sc.data_ptr(), x.data_ptr(), out.data_ptr(), (size_t)OC, (size_t)B,
                                  (size_t)IC, ws_ptr, (int)splitK);
+    }
     if (rc != 0) throw std::runtime_error(std::string("fp6mi_linear_native: ") + fp6mi_error_string(rc));
     return out;
 }
@@ -95,6 +105,6 @@ PYBIND11_MODULE(_fp6mi_torch, m)
     m.doc() = "torch tensors -> fp6mi C ABI";
     m.def("linear_forward_native", &linear_forward_native, pybind11::arg("EXPONENT"), pybind11::arg("MANTISSA"), pybind11::arg("in_feats"),
           pybind11::arg("native_weight"), pybind11::arg("scales"), pybind11::arg("OC"), pybind11::arg("splitK") = 1, pybind11::arg("out") = pybind11::none(),
-          pybind11::arg("workspace") = pybind11::none());
+          pybind11::arg("workspace") = pybind11::none(), pybind11::arg("group_exps") = pybind11::none());
     m.def("clear_workspaces", &clear_workspaces);
 }

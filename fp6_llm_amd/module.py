@@ -7,8 +7,8 @@ import numpy as np
 import torch
 
 from . import quant
-from . import (MI355X_CUS, heuristic_splitk_mi355x, linear_forward_native, native_bytes, to_native, weight_dequant_native_cuda,
-               weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu, weight_quantize_native_cuda)
+from . import (MI355X_CUS, group_exps_bytes, heuristic_splitk_mi355x, linear_forward_native, native_bytes, pack_group_exps, to_native,
+               weight_dequant_native_cuda, weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu, weight_quantize_native_cuda)
 
 _MAGIC = b"FP6MI\x00\x01\x00"   # name, NUL, layout version 1, reserved
 
@@ -33,6 +33,8 @@ class FPxLinear(torch.nn.Module):
         self.register_buffer("weight_native", torch.zeros(native_bytes(exponent, mantissa, out_features, in_features) // 4, dtype=torch.int32))
         self.register_buffer("scales", torch.ones(out_features, dtype=torch.float16))
         self.register_buffer("bias", bias)
+        # per-group exponents (one byte per row and 128 columns, in the kernels' order), or None for row scales only
+        self.register_buffer("group_exps", None)
 
     @classmethod
     def from_raw(cls, raw_int32, scales, exponent=3, mantissa=2, bias=None, split_k=None):
@@ -55,9 +57,16 @@ class FPxLinear(torch.nn.Module):
         return m
 
     @classmethod
-    def from_float(cls, weight, exponent=3, mantissa=2, bias=None, split_k=None):
+    def from_float(cls, weight, exponent=3, mantissa=2, bias=None, split_k=None, group_scales=False):
         """Quantizes a float [OC, IC] weight row-wise (round to nearest even, absmax scales) and packs it; a weight that
-        already lives on the GPU is quantized there (same bits as the host path)."""
+        already lives on the GPU is quantized there (same bits as the host path).  group_scales=True adds a power-of-two
+        factor per row and 128 columns (quant.quantize_groupwise, on the host), which the kernels apply for free."""
+        if group_scales:
+            codes, scales, exps = quant.quantize_groupwise(weight.detach().float().cpu().numpy(), exponent, mantissa)
+            raw = torch.from_numpy(quant.pack_raw(codes, exponent, mantissa))
+            m = cls.from_raw(raw, torch.from_numpy(scales), exponent, mantissa, bias, split_k)
+            m.group_exps = pack_group_exps(torch.from_numpy(exps), weight.shape[0], weight.shape[1])
+            return m.to(weight.device)
         if weight.device.type == "cuda" and weight.dtype in (torch.float16, torch.bfloat16, torch.float32):
             native, scales = weight_quantize_native_cuda(exponent, mantissa, weight.detach())
             m = cls(weight.shape[1], weight.shape[0], exponent, mantissa, bias, split_k).to(weight.device)
@@ -82,11 +91,15 @@ class FPxLinear(torch.nn.Module):
                 raise ValueError("fused layers must all have a bias or all have none")
             if l.weight_native.device != first.weight_native.device:
                 raise ValueError("fused layers must live on one device")
+            if (l.group_exps is None) != (first.group_exps is None):
+                raise ValueError("fused layers must all have group exponents or all have none")
         bias = None if first.bias is None else torch.cat([l.bias for l in layers])
         m = cls(first.in_features, sum(l.out_features for l in layers), first.exponent, first.mantissa, bias, split_k)
         m = m.to(first.weight_native.device)
         m.weight_native.copy_(torch.cat([l.weight_native for l in layers]))
         m.scales.copy_(torch.cat([l.scales for l in layers]))
+        if first.group_exps is not None:   # [row tile][K block][16][2] bytes: row tiles follow each other like the weights
+            m.group_exps = torch.cat([l.group_exps for l in layers])
         return m
 
     def forward(self, x):
@@ -95,7 +108,8 @@ class FPxLinear(torch.nn.Module):
         if x2.dtype != torch.float16:
             x2 = x2.half()
         if self.dequant_above is not None and x2.shape[0] >= self.dequant_above:
-            w16 = weight_dequant_native_cuda(self.exponent, self.mantissa, self.weight_native, self.scales, self.out_features, self.in_features)
+            w16 = weight_dequant_native_cuda(self.exponent, self.mantissa, self.weight_native, self.scales, self.out_features, self.in_features,
+                                             self.group_exps)
             y = torch.nn.functional.linear(x2, w16)
             del w16
             if self.bias is not None:
@@ -106,7 +120,7 @@ class FPxLinear(torch.nn.Module):
             sk = self._split_cache.get(x2.shape[0])
             if sk is None:
                 sk = self._split_cache[x2.shape[0]] = heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS)
-        y = linear_forward_native(self.exponent, self.mantissa, x2, self.weight_native, self.scales, self.out_features, sk)
+        y = linear_forward_native(self.exponent, self.mantissa, x2, self.weight_native, self.scales, self.out_features, sk, None, None, self.group_exps)
         if self.bias is not None:
             y = y + self.bias
         return y.reshape(*lead, self.out_features)
@@ -115,24 +129,33 @@ class FPxLinear(torch.nn.Module):
         return "in_features=%d, out_features=%d, format=e%dm%d" % (self.in_features, self.out_features, self.exponent, self.mantissa)
 
 
-def save_native(path, native_int32, scales, exponent, mantissa, out_features, in_features):
-    """One weight matrix in the native layout: magic, little-endian uint32 header length, JSON header, native bytes, fp16 scales."""
+def save_native(path, native_int32, scales, exponent, mantissa, out_features, in_features, group_exps=None):
+    """One weight matrix in the native layout: magic, little-endian uint32 header length, JSON header, native bytes, fp16 scales,
+    then the packed group exponents if the weight has them."""
     nat = native_int32.detach().cpu().contiguous().numpy()
     sc = scales.detach().cpu().contiguous().numpy().astype(np.float16)
     if nat.nbytes != native_bytes(exponent, mantissa, out_features, in_features) or sc.shape != (out_features,):
         raise ValueError("buffers do not match the stated shape")
+    ge = None
+    if group_exps is not None:
+        ge = group_exps.detach().cpu().contiguous().numpy()
+        if ge.dtype != np.uint8 or ge.size != group_exps_bytes(out_features, in_features):
+            raise ValueError("group_exps does not match the stated shape")
     header = json.dumps({"exponent": exponent, "mantissa": mantissa, "out_features": out_features, "in_features": in_features,
-                         "layout": "native-v1", "native_bytes": int(nat.nbytes)}).encode()
+                         "layout": "native-v1", "native_bytes": int(nat.nbytes), "group_exps_bytes": 0 if ge is None else int(ge.size)}).encode()
     with open(path, "wb") as f:
         f.write(_MAGIC)
         f.write(struct.pack("<I", len(header)))
         f.write(header)
         f.write(nat.tobytes())
         f.write(sc.tobytes())
+        if ge is not None:
+            f.write(ge.tobytes())
 
 
 def load_native(path):
-    """Returns (native int32 tensor, float16 scales, header dict).  Plain binary parsing; nothing in the file is executed."""
+    """Returns (native int32 tensor, float16 scales, header dict); the packed group exponents, if the file has them, are
+    hdr["group_exps"] (uint8 tensor).  Plain binary parsing; nothing in the file is executed."""
     with open(path, "rb") as f:
         if f.read(len(_MAGIC)) != _MAGIC:
             raise ValueError("%s is not a native FPx weight file (or has another layout version)" % path)
@@ -147,4 +170,12 @@ def load_native(path):
         sc = np.frombuffer(f.read(2 * hdr["out_features"]), dtype=np.float16)
         if nat.nbytes != want or sc.size != hdr["out_features"]:
             raise ValueError("file is truncated")
+        gbytes = int(hdr.get("group_exps_bytes", 0))
+        if gbytes:
+            if gbytes != group_exps_bytes(hdr["out_features"], hdr["in_features"]):
+                raise ValueError("header does not describe the group exponents of that shape")
+            ge = np.frombuffer(f.read(gbytes), dtype=np.uint8)
+            if ge.size != gbytes:
+                raise ValueError("file is truncated")
+            hdr["group_exps"] = torch.from_numpy(ge.copy())
     return torch.from_numpy(nat.copy()), torch.from_numpy(sc.copy()), hdr

@@ -57,6 +57,40 @@ def quantize_rowwise(weight, E=3, M=2):
     return quantize_codes(w / scale.astype(np.float64)[:, None], E, M), scale
 
 
+GROUP = 128   # columns per group exponent: a lane's share of a half K block in the native layout
+
+
+def quantize_groupwise(weight, E=3, M=2):
+    """weight [OC, IC] float -> (codes uint8 [OC, IC], scales float16 [OC], exps uint8 [OC, ceil(IC/128)]).
+    Two-level scaling: the row scale of quantize_rowwise, and per group of 128 columns the smallest power of two 2^(b-127),
+    112 <= b <= 127, that still holds the group's largest magnitude: weight ~ value(code) * 2^(b-127) * scale[row].
+    A group whose magnitudes are small next to the row maximum keeps up to 15 more bits of them than the row scale would."""
+    w = np.asarray(weight, dtype=np.float64)
+    OC, IC = w.shape
+    top = max_value(E, M)
+    scale = (np.abs(w).max(axis=1) / top).astype(np.float16)
+    scale = np.where(scale == 0, np.float16(1.0), scale).astype(np.float16)
+    groups = (IC + GROUP - 1) // GROUP
+    pad = np.zeros((OC, groups * GROUP))
+    pad[:, :IC] = np.abs(w)
+    gmax = pad.reshape(OC, groups, GROUP).max(axis=2) / scale.astype(np.float64)[:, None]     # in units of the row scale
+    with np.errstate(divide="ignore"):
+        k = np.ceil(np.log2(gmax / top))                       # smallest k with gmax <= top * 2^k (checked below: log2 rounds)
+    k = np.where(gmax > 0, k, -15.0)
+    k = np.where(gmax > top * np.exp2(k), k + 1, k)
+    k = np.where((k > -15) & (gmax <= top * np.exp2(k - 1)), k - 1, k)
+    k = np.clip(k, -15, 0).astype(np.int64)
+    factor = np.repeat(np.exp2(k.astype(np.float64)), GROUP, axis=1)[:, :IC] * scale.astype(np.float64)[:, None]
+    return quantize_codes(w / factor, E, M), scale, (k + 127).astype(np.uint8)
+
+
+def dequantize_grouped(codes, scales, exps, E=3, M=2):
+    """float64 value(code) * 2^(b-127) * scale, for checks."""
+    c = np.asarray(codes)
+    f = np.repeat(np.exp2(np.asarray(exps, dtype=np.float64) - 127.0), GROUP, axis=1)[:, :c.shape[1]]
+    return dequantize_codes(c, scales, E, M) * f
+
+
 def pack_raw(codes, E=3, M=2):
     """codes uint8 [OC, IC] -> int32 [OC, IC/32*x]: each row an MSB-first bitstream carried in little-endian int32 words,
     the raw weight format of the reference (fp6_llm/csrc/utils/common.h:4-19; worked example

@@ -127,6 +127,26 @@ int fp6mi_dequant_native_gpu(int E, int Mbits, void *stream, void *out_f16_dev, 
 int fp6mi_quantize_native_gpu(int E, int Mbits, void *stream, void *native_dev, void *scales_f16_dev,
                               const void *weights_dev, int dtype, size_t M, size_t K);
 
+/* ---------------------------------------------------------------------------------- per-group scales (beyond the reference)
+ * The reference scales per output row only (fp6_llm/csrc/fp6_linear.cuh:24, one half per row).  Here a weight matrix may
+ * carry, besides its row scales, one exponent byte b per (row, group of 128 columns): the weights of the group count
+ * value * 2^(b-127) * scale[row]  (b is the E8M0 scale type of the OCP MX formats; 127 = factor 1).  The gfx950 conversion
+ * instruction applies the power of two while it converts, so a grouped GEMM runs at the speed of an ungrouped one.
+ * b must keep value * 2^(b-127) inside fp16 (112 <= b <= 135 always does); the quantizer of the Python package emits
+ * 112..127.  `exps` is row-major [M][ceil(K/128)] bytes; the kernels read the "native" order produced by
+ * fp6mi_pack_group_exps: fp6mi_group_exps_bytes(M, K) bytes, M % 16 == 0, K % 64 == 0. */
+size_t fp6mi_group_exps_bytes(size_t M, size_t K);
+int    fp6mi_pack_group_exps(void *native_exps, const void *exps, size_t M, size_t K);
+/* fp6mi_dequant with group exponents (host; raw weights, exps row-major). */
+int fp6mi_dequant_grouped(int E, int Mbits, void *out_f16, const void *raw, size_t M, size_t K, const void *scales_f16,
+                          const void *exps);
+/* fp6mi_linear_native / fp6mi_dequant_native_gpu with group exponents (device pointer, native order, 2-byte aligned). */
+int fp6mi_linear_native_grouped(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
+                                const void *group_exps_native, const void *B_f16, void *C_f16, size_t M, size_t N, size_t K,
+                                float *workspace, int splitK);
+int fp6mi_dequant_native_grouped_gpu(int E, int Mbits, void *stream, void *out_f16_dev, const void *W_native_dev,
+                                     const void *scales_f16_dev, const void *group_exps_native_dev, size_t M, size_t K);
+
 #ifdef __cplusplus
 }
 #endif

@@ -290,6 +290,18 @@ def dequant_from_definition(codes, scale, E=3, M=2):
     return prod.astype(np.float16)
 
 
+def dequant_grouped_from_definition(codes, scale, exps, E=3, M=2):
+    """fp16_rn(value(code) * 2^(b-127) * scale) with one exponent byte b per (row, 128 columns): the definition of this
+    build's per-group scales.  The reference has no per-group scales (one half per row, fp6_llm/csrc/fp6_linear.cuh:24), so
+    there is no reference behaviour to pin this against: PARITY UNPINNED, the definition itself is the arbiter."""
+    tab = value_table(E, M)
+    codes = np.asarray(codes)
+    f = np.repeat(np.exp2(np.asarray(exps, dtype=np.float64) - 127.0), 128, axis=1)[:, :codes.shape[1]]
+    prod = tab[codes] * f * np.asarray(scale, dtype=np.float16).astype(np.float64)[:, None]   # exact in float64
+    with np.errstate(over="ignore"):
+        return prod.astype(np.float16)
+
+
 def gemm_f64(wdq, x):
     """float64 accumulation of the dequantized weights: the arbiter for GEMM tolerance checks. Returns float64 [N, OC]."""
     return np.asarray(x, dtype=np.float64) @ np.asarray(wdq, dtype=np.float64).T

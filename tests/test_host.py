@@ -294,6 +294,78 @@ def test_native_weight_file_round_trip(tmp_path):
         module.load_native(path)
 
 
+# ------------------------------------------------------------------------------------------------ per-group exponents
+def _grouped_problem(seed, OC, IC, E, M):
+    """Gaussian weights whose groups of 128 columns differ in magnitude by powers of e, so that the exponents vary."""
+    rng = np.random.default_rng(seed)
+    spread = np.exp(rng.normal(0, 1.5, (OC, (IC + 127) // 128))).repeat(128, axis=1)[:, :IC]
+    return synth.normal(seed, (OC, IC)) * spread
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_groupwise_quantizer(E, M):
+    OC, IC = 64, 320   # the last group has 64 columns
+    w = _grouped_problem(31, OC, IC, E, M)
+    codes, sc, ex = quant.quantize_groupwise(w, E, M)
+    top = quant.max_value(E, M)
+    assert ex.dtype == np.uint8 and ex.shape == (OC, 3) and ex.min() >= 112 and ex.max() == 127 and len(np.unique(ex)) > 3
+    _, sc_row = quant.quantize_rowwise(w, E, M)
+    assert (sc == sc_row).all()                                  # the row scale is the row-wise one
+    for g in range(3):
+        blockmax = np.abs(w[:, 128 * g:128 * g + 128]).max(axis=1) / sc.astype(np.float64)
+        f = np.exp2(ex[:, g].astype(np.float64) - 127)
+        # the group fits under its factor (the row's largest group only up to the rounding of the fp16 row scale, like row-wise) ...
+        assert ((blockmax <= top * f) | ((ex[:, g] == 127) & (blockmax <= top * (1 + 2.0 ** -10)))).all()
+        assert ((blockmax > top * f / 2) | (ex[:, g] == 112)).all()   # ... and would not fit under half of it
+    deq = quant.dequantize_grouped(codes, sc, ex, E, M)
+    rw_codes, _ = quant.quantize_rowwise(w, E, M)
+    assert np.abs(deq - w).mean() < np.abs(quant.dequantize_codes(rw_codes, sc, E, M) - w).mean()
+    # weights without spread between groups of a row's own maximum group keep factor 1 there
+    assert (ex.max(axis=1) == 127).all()
+    # a zero matrix: scale 1, any exponent, all codes zero magnitude
+    c0, s0, e0 = quant.quantize_groupwise(np.zeros((16, 128)), E, M)
+    assert (s0 == 1).all() and (c0 & ((1 << (E + M)) - 1) == 0).all() and e0.shape == (16, 1)
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_grouped_dequant_and_exponent_packing(E, M):
+    OC, IC = 64, 320
+    codes, sc, ex = quant.quantize_groupwise(_grouped_problem(32, OC, IC, E, M), E, M)
+    raw = torch.from_numpy(quant.pack_raw(codes, E, M))
+    dq = fp6.weight_dequant_grouped_cpu(E, M, raw, torch.from_numpy(sc), torch.from_numpy(ex)).numpy()
+    assert (dq.view(np.uint16) == oracle.dequant_grouped_from_definition(codes, sc, ex, E, M).view(np.uint16)).all()
+    ones = torch.full((OC, 3), 127, dtype=torch.uint8)               # factor 1 everywhere = the reference's dequantizer
+    assert torch.equal(fp6.weight_dequant_grouped_cpu(E, M, raw, torch.from_numpy(sc), ones),
+                       fp6.weight_dequant_eXmY_cpu(E, M, raw, torch.from_numpy(sc)))
+    # packed order, from its definition: [row tile][K block][row in tile][half]; halves beyond IC hold 127
+    nat = fp6.pack_group_exps(torch.from_numpy(ex), OC, IC).numpy()
+    assert nat.size == fp6.group_exps_bytes(OC, IC) == (OC // 16) * 2 * 32
+    for (R, U, m, h) in [(0, 0, 0, 0), (3, 0, 15, 1), (2, 1, 7, 0), (1, 1, 9, 1)]:
+        want = ex[16 * R + m, 2 * U + h] if 2 * U + h < 3 else 127
+        assert nat[((R * 2 + U) * 16 + m) * 2 + h] == want
+    with pytest.raises(ValueError):
+        fp6.pack_group_exps(torch.from_numpy(ex[:, :2].copy()), OC, IC)
+
+
+def test_grouped_weight_file_and_fused_layers(tmp_path):
+    from fp6_llm_amd import module
+    E, M = 2, 1
+    ws = [torch.from_numpy(_grouped_problem(40 + i, oc, 384, E, M)).float() for i, oc in enumerate((256, 512))]
+    parts = [module.FPxLinear.from_float(w, E, M, group_scales=True) for w in ws]
+    whole = module.FPxLinear.from_float(torch.cat(ws), E, M, group_scales=True)
+    fused = module.FPxLinear.fused(parts)
+    assert fused.group_exps is not None and torch.equal(fused.group_exps, whole.group_exps)
+    assert torch.equal(fused.weight_native, whole.weight_native) and torch.equal(fused.scales, whole.scales)
+    with pytest.raises(ValueError):
+        module.FPxLinear.fused([parts[0], module.FPxLinear.from_float(ws[1], E, M)])
+    path = str(tmp_path / "g.fp6mi")
+    module.save_native(path, whole.weight_native, whole.scales, E, M, 768, 384, whole.group_exps)
+    nat2, sc2, hdr = module.load_native(path)
+    assert torch.equal(nat2, whole.weight_native) and torch.equal(sc2, whole.scales) and torch.equal(hdr["group_exps"], whole.group_exps)
+    module.save_native(path, whole.weight_native, whole.scales, E, M, 768, 384)
+    assert "group_exps" not in module.load_native(path)[2]
+
+
 def test_module_construction_routes_agree():
     from fp6_llm_amd import module
     raw, sc = _problem(22, 256, 128, 3, 2)
