@@ -57,11 +57,11 @@ HEADLINE = "fp6_4096x4096_bs8"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
 # for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {
-    "fp6_4096x4096_bs8": 13244911,
-    "fp6_8192x8192_bs8": 51570043,
-    "fp5_8192x8192_bs8": 43196662,
-    "fp6_28672x8192_bs32": 182255785,
-    "fp6_8192x8192_bs512": 125981259,
+    "fp6_4096x4096_bs8": 13239792,
+    "fp6_8192x8192_bs8": 51576185,
+    "fp5_8192x8192_bs8": 43183355,
+    "fp6_28672x8192_bs32": 182260903,
+    "fp6_8192x8192_bs512": 125992391,
 }
 
 

@@ -233,10 +233,12 @@ def weight_dequant_native_cuda(EXPONENT, MANTISSA, native_weight, fp16_scale, OC
 _QUANT_DTYPES = {torch.float16: 0, torch.bfloat16: 1, torch.float32: 2}
 
 
-def weight_quantize_native_cuda(EXPONENT, MANTISSA, weight):
+def weight_quantize_native_cuda(EXPONENT, MANTISSA, weight, group_scales=False):
     """Float weights [OC, IC] (fp16, bf16 or fp32) on the GPU -> (native-layout int32 tensor, fp16 scales [OC]) on the same GPU:
     per-row absmax scales, round to nearest with ties to the even code, clamped at the format maximum.  Gives the same
-    bits as quant.quantize_rowwise + quant.pack_raw + weight_prepacking_native_cpu on the host, without leaving the device."""
+    bits as quant.quantize_rowwise + quant.pack_raw + weight_prepacking_native_cpu on the host, without leaving the device.
+    group_scales=True also chooses a power-of-two factor per row and 128 columns and returns (native, scales, group_exps),
+    the same bits as quant.quantize_groupwise + pack_group_exps."""
     _bits(EXPONENT, MANTISSA)
     if weight.device.type != "cuda" or weight.dim() != 2 or weight.dtype not in _QUANT_DTYPES:
         raise ValueError("weight must be a 2-D fp16, bf16 or fp32 tensor on the GPU")
@@ -248,6 +250,12 @@ def weight_quantize_native_cuda(EXPONENT, MANTISSA, weight):
     scales = torch.empty(OC, dtype=torch.float16, device=weight.device)
     with torch.cuda.device(weight.device):
         stream = torch.cuda.current_stream().cuda_stream
+        if group_scales:
+            gexp = torch.empty(group_exps_bytes(OC, IC), dtype=torch.uint8, device=weight.device)
+            _lib.check(_lib.lib().fp6mi_quantize_native_grouped_gpu(EXPONENT, MANTISSA, stream, native.data_ptr(), scales.data_ptr(), gexp.data_ptr(),
+                                                                    weight.data_ptr(), _QUANT_DTYPES[weight.dtype], OC, IC),
+                       "fp6mi_quantize_native_grouped_gpu")
+            return native, scales, gexp
         _lib.check(_lib.lib().fp6mi_quantize_native_gpu(EXPONENT, MANTISSA, stream, native.data_ptr(), scales.data_ptr(), weight.data_ptr(),
                                                         _QUANT_DTYPES[weight.dtype], OC, IC), "fp6mi_quantize_native_gpu")
     return native, scales

@@ -49,6 +49,7 @@ def lib():
         "fp6mi_dequant_grouped": (ci, [ci, ci, vp, vp, sz, sz, vp, vp]),
         "fp6mi_linear_native_grouped": (ci, [ci, ci, vp, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci]),
         "fp6mi_dequant_native_grouped_gpu": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz]),
+        "fp6mi_quantize_native_grouped_gpu": (ci, [ci, ci, vp, vp, vp, vp, vp, ci, sz, sz]),
     }
     for name, (res, args) in sigs.items():
         fn = getattr(L, name)
@@ -63,7 +64,7 @@ EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_prepack_ref", "fp6mi_d
             "fp6mi_heuristic_splitk", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_twin_evict", "fp6mi_twin_clear",
             "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch",
             "fp6mi_group_exps_bytes", "fp6mi_pack_group_exps", "fp6mi_dequant_grouped", "fp6mi_linear_native_grouped",
-            "fp6mi_dequant_native_grouped_gpu"]
+            "fp6mi_dequant_native_grouped_gpu", "fp6mi_quantize_native_grouped_gpu"]
 
 
 def check(code, where):

@@ -706,8 +706,11 @@ template <int FM> __device__ __forceinline__ uint32_t nearest_magnitude(double a
     return lo;
 }
 
+// gexp (native order) non-null: besides the row scale every group of 128 columns of a row gets the smallest factor 2^k,
+// -15 <= k <= 0, that still holds its largest magnitude, stored as the byte 127 + k, and its codes are chosen against
+// scale * 2^k.  A wavefront's lanes (m, q = 0..3) hold the group's 128 values between them, 32 each.
 template <int FM, typename T>
-__global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ native, const half_t *__restrict__ scales,
+__global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ native, const half_t *__restrict__ scales, uint8_t *__restrict__ gexp,
                                                       const T *__restrict__ Wf, uint32_t M, uint32_t K, uint32_t units, double max_value)
 {
     const int      lane = threadIdx.x & 63;
@@ -718,15 +721,35 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
     const uint32_t row = R * 16 + m;
     const double   sc = (double)(float)scales[row];
     const T       *p = Wf + (size_t)row * K;
-    uint8_t        c[64];
+    double         factor[2] = { sc, sc };
+    if (gexp) { // uniform
+        for (int h = 0; h < 2; h++) {
+            float amax = 0.f;
+            for (int s = 4 * h; s < 4 * h + 4; s++) {
+                const uint32_t k0 = U * 256 + 32 * s + 8 * q;
+                for (int j = 0; j < 8; j++)
+                    if (k0 + j < K) amax = fmaxf(amax, fabsf(to_float<T>(p[k0 + j])));
+            }
+            amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+            amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+            const double gmax = (double)amax / sc;
+            int          k = -15;
+            while (k < 0 && !(gmax <= scalbn(max_value, k))) k++;
+            if (U * 256 + 128 * h >= K) k = 0; // a half block beyond K: factor 1 by convention
+            factor[h] = scalbn(sc, k);
+            if (q == 0) gexp[((size_t)blk * 16 + m) * 2 + h] = (uint8_t)(127 + k);
+        }
+    }
+    uint8_t c[64];
 #pragma unroll 1
     for (int s = 0; s < 8; s++) {
         const uint32_t k0 = U * 256 + 32 * s + 8 * q;
+        const double   f = factor[s >> 2];
         for (int j = 0; j < 8; j++) {
             uint32_t code = 0;
             if (k0 + j < K) {
                 float  w = to_float<T>(p[k0 + j]);
-                double a = fabs((double)w / sc);
+                double a = fabs((double)w / f);
                 if (!(a <= max_value)) a = max_value; // clamps, and sends NaN to the maximum like a saturating cast
                 code = nearest_magnitude<FM>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (Fmt<FM>::bits - 1));
             }
@@ -836,7 +859,7 @@ template <int FM> int op_dequant(void *stream, void *out, const void *W, const v
 }
 
 // dtype: 0 = fp16, 1 = bf16, 2 = fp32
-template <int FM> int op_quantize(void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K)
+template <int FM> int op_quantize(void *stream, void *native, void *scales, void *gexp, const void *weights, int dtype, size_t M, size_t K)
 {
     const uint32_t   units = (uint32_t)((K + 255) / 256);
     const size_t     blocks = (M / 16) * units;
@@ -848,7 +871,8 @@ template <int FM> int op_quantize(void *stream, void *native, void *scales, cons
     auto             run = [&](auto *typed) {
         typedef std::remove_cv_t<std::remove_pointer_t<decltype(typed)>> T;
         hipLaunchKernelGGL(quant_row_scales<T>, grid_rows, dim3(256), 0, st, sc, typed, (uint32_t)M, (uint32_t)K, max_value);
-        hipLaunchKernelGGL((quant_to_native<FM, T>), grid_blocks, dim3(256), 0, st, nat, sc, typed, (uint32_t)M, (uint32_t)K, units, max_value);
+        hipLaunchKernelGGL((quant_to_native<FM, T>), grid_blocks, dim3(256), 0, st, nat, sc, static_cast<uint8_t *>(gexp), typed, (uint32_t)M,
+                           (uint32_t)K, units, max_value);
     };
     if (dtype == 0)
         run(static_cast<const half_t *>(weights));

@@ -23,7 +23,7 @@ struct FormatOps {
                 size_t N, size_t K, int splitK);
     int (*relayout)(void *stream, void *native, const void *packed_ref, size_t M, size_t K);
     int (*dequant)(void *stream, void *out_f16, const void *W, const void *sc, const void *gexp, size_t M, size_t K);
-    int (*quantize)(void *stream, void *native, void *scales, const void *weights, int dtype, size_t M, size_t K);
+    int (*quantize)(void *stream, void *native, void *scales, void *gexp, const void *weights, int dtype, size_t M, size_t K); // gexp may be null
 };
 const FormatOps &format_ops_32(), &format_ops_22(), &format_ops_23(), &format_ops_21(); // named by 10*E + M
 inline const FormatOps *ops_for(int E, int Mbits)

@@ -60,7 +60,15 @@ class FPxLinear(torch.nn.Module):
     def from_float(cls, weight, exponent=3, mantissa=2, bias=None, split_k=None, group_scales=False):
         """Quantizes a float [OC, IC] weight row-wise (round to nearest even, absmax scales) and packs it; a weight that
         already lives on the GPU is quantized there (same bits as the host path).  group_scales=True adds a power-of-two
-        factor per row and 128 columns (quant.quantize_groupwise, on the host), which the kernels apply for free."""
+        factor per row and 128 columns (quant.quantize_groupwise), which the conversion instruction applies."""
+        on_gpu = weight.device.type == "cuda" and weight.dtype in (torch.float16, torch.bfloat16, torch.float32)
+        if group_scales and on_gpu:
+            native, scales, gexp = weight_quantize_native_cuda(exponent, mantissa, weight.detach(), True)
+            m = cls(weight.shape[1], weight.shape[0], exponent, mantissa, bias, split_k).to(weight.device)
+            m.weight_native.copy_(native)
+            m.scales.copy_(scales)
+            m.group_exps = gexp
+            return m
         if group_scales:
             codes, scales, exps = quant.quantize_groupwise(weight.detach().float().cpu().numpy(), exponent, mantissa)
             raw = torch.from_numpy(quant.pack_raw(codes, exponent, mantissa))

@@ -146,6 +146,11 @@ int fp6mi_linear_native_grouped(int E, int Mbits, void *stream, const void *W_na
                                 float *workspace, int splitK);
 int fp6mi_dequant_native_grouped_gpu(int E, int Mbits, void *stream, void *out_f16_dev, const void *W_native_dev,
                                      const void *scales_f16_dev, const void *group_exps_native_dev, size_t M, size_t K);
+/* fp6mi_quantize_native_gpu that also chooses the group exponents: per group the smallest 2^(b-127), 112 <= b <= 127, that
+ * holds the group's largest |weight| / scale[row]; codes are rounded against scale * 2^(b-127).  Writes
+ * fp6mi_group_exps_bytes(M, K) bytes in native order. */
+int fp6mi_quantize_native_grouped_gpu(int E, int Mbits, void *stream, void *native_dev, void *scales_f16_dev,
+                                      void *group_exps_native_dev, const void *weights_dev, int dtype, size_t M, size_t K);
 
 #ifdef __cplusplus
 }

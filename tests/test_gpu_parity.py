@@ -518,6 +518,24 @@ def test_grouped_gemm_and_dequant(E, M, OC, IC, BS, splitK):
     assert L.fp6mi_linear_native_grouped(E, M, None, native.data_ptr(), scd.data_ptr(), None, xd.data_ptr(), out.data_ptr(), OC, BS, IC, None, 1) == -3
 
 
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("OC,IC", [(256, 512), (512, 320)])
+def test_device_groupwise_quantizer_matches_host_bits(E, M, dtype, OC, IC):
+    """Same scales, exponents and codes as quant.quantize_groupwise + pack_group_exps; K = 320 leaves the last group half
+    full and the last half block beyond K."""
+    print("case device group quantizer", E, M, dtype, OC, IC, flush=True)
+    w = _awkward_weights(43, OC, IC, dtype)
+    spread = np.exp(np.random.default_rng(3).normal(0, 2.0, (OC, (IC + 127) // 128))).repeat(128, axis=1)[:, :IC]
+    spread[:8] = 1.0                                   # keep the special rows (zeros, ties, subnormal scale) as they are
+    w = (w.float() * torch.from_numpy(spread).float()).to(dtype)
+    native, scales, gexp = fp6.weight_quantize_native_cuda(E, M, w.to(DEV), group_scales=True)
+    codes, sc_host, ex_host = quant.quantize_groupwise(w.float().numpy().astype(np.float64), E, M)
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), sc_host.view(np.uint16))
+    assert torch.equal(gexp.cpu(), fp6.pack_group_exps(torch.from_numpy(ex_host), OC, IC))
+    assert torch.equal(native.cpu(), fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))))
+
+
 def test_grouped_module_forward_and_prefill_route():
     from fp6_llm_amd import module
     E, M, OC, IC = 2, 1, 512, 1024
