@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """The linear layers of one transformer decoder layer at decode batch sizes, FPx weights against FP16 weights.
 
-    python examples/decode_layer.py [--model 7b|70b] [--format 6|5|4] [--batch 1,8,32]
+    python examples/decode_layer.py [--model 7b|70b] [--format 6|5|4] [--batch 1,8,32] [--group-scales]
 
 Builds the four GEMMs of a LLaMA-shaped layer as `FPxLinear` modules -- Q, K and V fused into one launch and gate and up
 into another with `FPxLinear.fused` -- quantizes random weights on the GPU, captures one pass over the four layers into a
@@ -54,6 +54,7 @@ def main():
     ap.add_argument("--model", default="7b", choices=sorted(SHAPES))
     ap.add_argument("--format", type=int, default=6, choices=(4, 5, 6), help="6 = FP6_e3m2, 5 = FP5_e2m2, 4 = FP4_e2m1")
     ap.add_argument("--batch", default="1,8,32")
+    ap.add_argument("--group-scales", action="store_true", help="a power-of-two factor per row and 128 columns besides the row scales")
     args = ap.parse_args()
     dims = SHAPES[args.model]
     H, KV, F = dims["hidden"], dims["kv"], dims["mlp"]
@@ -66,8 +67,8 @@ def main():
         g = torch.Generator(device=dev).manual_seed(copy)
         w = lambda o, i: torch.randn(o, i, generator=g, device=dev, dtype=torch.float16) * 0.02   # noqa: E731
         wq, wk, wv, wo, wg, wu, wd = w(H, H), w(KV, H), w(KV, H), w(H, H), w(F, H), w(F, H), w(H, F)
-        fpx = dict(qkv=FPxLinear.fused([FPxLinear.from_float(t, E, M) for t in (wq, wk, wv)]), o=FPxLinear.from_float(wo, E, M),
-                   gate_up=FPxLinear.fused([FPxLinear.from_float(t, E, M) for t in (wg, wu)]), down=FPxLinear.from_float(wd, E, M))
+        q = lambda t: FPxLinear.from_float(t, E, M, group_scales=args.group_scales)   # noqa: E731
+        fpx = dict(qkv=FPxLinear.fused([q(t) for t in (wq, wk, wv)]), o=q(wo), gate_up=FPxLinear.fused([q(t) for t in (wg, wu)]), down=q(wd))
         f16 = dict(qkv=torch.cat([wq, wk, wv]), o=wo, gate_up=torch.cat([wg, wu]), down=wd)
         return fpx, f16
 
