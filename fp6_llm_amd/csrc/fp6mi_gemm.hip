@@ -15,6 +15,7 @@
 // applied once to the FP32 sums instead of to every weight.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <type_traits>
 
 #include "fp6mi_internal.h"
@@ -781,12 +782,17 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *gexp,
     constexpr size_t lds_bytes = x_bytes > red_bytes ? x_bytes : red_bytes;
     static_assert(lds_bytes <= 160 * 1024, "tile does not fit in LDS");
     if (M % TM) return FP6MI_ERR_SHAPE;
-    static bool attr_set = false; // idempotent, so a race between host threads is harmless
-    if (!attr_set && lds_bytes > 48 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, GS, NT, RT, WR, WK>),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-        if (e != hipSuccess) return (int)e;
-        attr_set = true;
+    if (lds_bytes > 48 * 1024) { // the attribute belongs to the device's copy of the kernel: once per device
+        static std::atomic<uint64_t> attr_set{ 0 }; // bit d: done on device d; setting it twice is harmless, so no lock
+        int                          dev = 0;
+        if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+        const uint64_t bit = dev < 64 ? 1ull << dev : 0;
+        if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, GS, NT, RT, WR, WK>),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+            if (e != hipSuccess) return (int)e;
+            attr_set.fetch_or(bit, std::memory_order_relaxed);
+        }
     }
     uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
     size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
