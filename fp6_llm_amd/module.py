@@ -17,8 +17,9 @@ class FPxLinear(torch.nn.Module):
     """y = x @ dequant(W)^T (+ bias) with W held in the native gfx950 layout.  Weights are buffers, not parameters:
     the layer is inference-only, like the kernels."""
 
-    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None, dequant_above=None):
-        """dequant_above: batch size from which forward() dequantizes the weights to a temporary fp16 matrix on the GPU and calls
+    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None, dequant_above=None, group_scales=False):
+        """group_scales: the layer also holds one exponent byte per row and 128 columns (factor 1 until weights are loaded).
+        dequant_above: batch size from which forward() dequantizes the weights to a temporary fp16 matrix on the GPU and calls
         the FP16 library GEMM instead (prefill).  The mixed-input kernel wins while the GEMM is bound by weight bytes; from a
         couple of thousand rows the FP16 library runs 1.3-1.4 PFLOP/s against its 0.9-1.0 (measured at 8192 x 8192), which
         pays for the dequantization pass.  None (default) never does: the temporary costs 2 bytes per weight."""
@@ -34,7 +35,7 @@ class FPxLinear(torch.nn.Module):
         self.register_buffer("scales", torch.ones(out_features, dtype=torch.float16))
         self.register_buffer("bias", bias)
         # per-group exponents (one byte per row and 128 columns, in the kernels' order), or None for row scales only
-        self.register_buffer("group_exps", None)
+        self.register_buffer("group_exps", torch.full((group_exps_bytes(out_features, in_features),), 127, dtype=torch.uint8) if group_scales else None)
 
     @classmethod
     def from_raw(cls, raw_int32, scales, exponent=3, mantissa=2, bias=None, split_k=None):

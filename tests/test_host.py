@@ -358,6 +358,12 @@ def test_grouped_weight_file_and_fused_layers(tmp_path):
     assert torch.equal(fused.weight_native, whole.weight_native) and torch.equal(fused.scales, whole.scales)
     with pytest.raises(ValueError):
         module.FPxLinear.fused([parts[0], module.FPxLinear.from_float(ws[1], E, M)])
+    # a layer built empty with group_scales=True takes the state of a quantized one
+    blank = module.FPxLinear(384, 768, E, M, group_scales=True)
+    assert (blank.group_exps == 127).all()
+    blank.load_state_dict(whole.state_dict())
+    assert torch.equal(blank.group_exps, whole.group_exps) and torch.equal(blank.weight_native, whole.weight_native)
+    assert "group_exps" not in module.FPxLinear(384, 768, E, M).state_dict()
     path = str(tmp_path / "g.fp6mi")
     module.save_native(path, whole.weight_native, whole.scales, E, M, 768, 384, whole.group_exps)
     nat2, sc2, hdr = module.load_native(path)
