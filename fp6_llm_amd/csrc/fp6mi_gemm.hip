@@ -130,10 +130,11 @@ template <bool GS> __device__ __forceinline__ float group_factor(uint32_t g, int
     else
         return 1.0f;
 }
-template <bool GS> __device__ __forceinline__ uint32_t load_group_exps(const uint8_t *gexp_block, int lane)
+// block = index of the 16x256 block counted from `gexp` (32 bytes each); nothing is computed or read without group exponents
+template <bool GS> __device__ __forceinline__ uint32_t load_group_exps(const uint8_t *gexp, size_t block, int lane)
 {
     if constexpr (GS)
-        return *reinterpret_cast<const uint16_t *>(gexp_block + 2 * (lane & 15));
+        return *reinterpret_cast<const uint16_t *>(gexp + block * 32 + 2 * (lane & 15));
     else
         return 0;
 }
@@ -188,7 +189,7 @@ __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t 
 #pragma unroll
     for (int r = 0; r < RT; r++) {
         st.w[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
-        st.g[r] = load_group_exps<GS>(ggroup + ((size_t)r * units + u) * 32, lane);
+        st.g[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
     }
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
             for (int r = 0; r < RT; r++) {
                 dst[r]  = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
-                gdst[r] = load_group_exps<GS>(ggroup + ((size_t)r * units + u) * 32, lane);
+                gdst[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
             }
         }
     };
@@ -523,7 +524,7 @@ __global__ __launch_bounds__(256) void dequant_native(half_t *__restrict__ out, 
     const int      m = lane & 15, q = lane >> 4;
     WFrag<FM>      wf = load_wfrag<FM>(W + (size_t)blk * Fmt<FM>::block_bytes, lane);
     AOps<FM>       a;
-    convert<FM, GS>(wf, a, load_group_exps<GS>(gexp + (size_t)blk * 32, lane));
+    convert<FM, GS>(wf, a, load_group_exps<GS>(gexp, blk, lane));
     const half_t sc = scales[R * 16 + m], post = (half_t)Fmt<FM>::post_scale;
 #pragma unroll
     for (int s = 0; s < 8; s++) {
