@@ -8,7 +8,13 @@ launches after a warm-up; the FP16 GEMM of the same shape on the same GPU (torch
 output, i.e. hipBLASLt) is timed the same way.  Prints time, TFLOP/s = 2*OC*IC*BS/t, the speed-up, and the error of the
 FPx result against the FP16 GEMM (mean|err| / mean|ref|, the reference's figure) and against an FP32 matmul of the
 dequantized weights (max |err| / max(|ref|, rms ref)).  --splitK 0 asks the engine's heuristic.
-Eager launches include Python and launch overhead (several microseconds each); bench.py replays HIP graphs instead."""
+Eager launches include Python and launch overhead (several microseconds each); bench.py replays HIP graphs instead.
+
+    python -m fp6_llm_amd.kernel_test --suite llama2-70b [--BS 1,8,32] [--EXP 3 --MAN 2]
+
+runs the shape lists of the reference's run scripts (tests/python/run.sh:33-34, tests/cpp/run.sh:7-8,14-15,22-23) one after
+the other, each at the batch sizes given (default: the scripts' own 1..64) with the engine's split-K, and prints one summary
+line per GEMM."""
 import argparse
 import sys
 
@@ -65,17 +71,45 @@ def run(OC, IC, BS, splitK=0, EXP=3, MAN=2, repeat=1000, warmup=10, seed=0, out=
     return res
 
 
+# (OC, IC) lists of the reference's run scripts
+SUITES = {
+    "llama2-70b": [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)],                                   # tests/python/run.sh:33-34
+    "llama1-65b": [(13824, 5120), (5120, 13824), (22016, 8192), (8192, 22016)],                                  # tests/cpp/run.sh:7-8
+    "opt": [(21504, 7168), (7168, 7168), (28672, 7168), (7168, 28672), (27648, 9216), (9216, 9216), (36864, 9216), (9216, 36864),
+            (36864, 12288), (12288, 12288), (49152, 12288), (12288, 49152)],                                     # tests/cpp/run.sh:14-15
+    "llama1": [(12288, 4096), (4096, 4096), (11008, 4096), (4096, 11008), (15360, 5120), (5120, 5120), (13824, 5120), (5120, 13824),
+               (19968, 6656), (6656, 6656), (17920, 6656), (6656, 17920), (24576, 8192), (8192, 8192), (22016, 8192), (8192, 22016)],  # :22-23
+}
+
+
+def run_suite(name, batches, EXP, MAN, repeat, out=sys.stdout):
+    import io
+    rows = []
+    for (OC, IC) in SUITES[name]:
+        for BS in batches:
+            r = run(OC, IC, BS, 0, EXP, MAN, repeat, out=io.StringIO())
+            rows.append(r)
+            print("OC=%6d IC=%6d BS=%4d splitK=%d  FPx %8.4f ms %7.1f TFLOP/s   fp16 %8.4f ms   speed-up %5.2f   max rel err %.2e"
+                  % (OC, IC, BS, r["splitK"], r["fpx_ms"], r["fpx_tflops"], r["fp16_ms"], r["speedup"], r["max_rel_err_vs_fp32"]), file=out, flush=True)
+    return rows
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description="One FPx x FP16 GEMM: (OC, IC) weights times (BS, IC) activations -> (BS, OC).")
     ap.add_argument("--OC", type=int, default=4096, help="rows of the weight matrix (multiple of 256)")
     ap.add_argument("--IC", type=int, default=4096, help="columns of the weight matrix (multiple of 64)")
-    ap.add_argument("--BS", type=int, default=32, help="batch size")
+    ap.add_argument("--BS", default="32", help="batch size (a comma-separated list with --suite)")
+    ap.add_argument("--suite", choices=sorted(SUITES), help="run a shape list of the reference's run scripts instead of one GEMM")
     ap.add_argument("--splitK", type=int, default=0, help="split of the K dimension; 0 = the engine's heuristic")
     ap.add_argument("--EXP", type=int, default=3, choices=(2, 3), help="exponent bits")
     ap.add_argument("--MAN", type=int, default=2, choices=(1, 2, 3), help="mantissa bits (e3m2, e2m2, e2m3 and e2m1 exist)")
     ap.add_argument("--repeat", type=int, default=1000)
     a = ap.parse_args(argv)
-    run(a.OC, a.IC, a.BS, a.splitK, a.EXP, a.MAN, a.repeat)
+    batches = [int(b) for b in str(a.BS).split(",")]
+    if a.suite:
+        run_suite(a.suite, batches if "," in str(a.BS) or a.BS != "32" else [1, 2, 4, 8, 16, 32, 64], a.EXP, a.MAN, min(a.repeat, 200))
+        return
+    run(a.OC, a.IC, batches[0], a.splitK, a.EXP, a.MAN, a.repeat)
 
 
 if __name__ == "__main__":

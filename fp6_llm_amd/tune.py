@@ -43,7 +43,7 @@ GRID_M = [1024, 2048, 3072, 4096, 5120, 6144, 8192, 10240, 11008, 12288, 14336, 
 GRID_K = [2048, 4096, 5120, 8192, 11008, 14336, 28672]
 GRID_N_SMALL = [1, 4, 8, 12, 16]
 GRID_N_LARGE = [24, 32, 48, 64, 96, 128, 256, 512, 1024, 2048]
-MAX_WEIGHTS = 240 * 1000 * 1000   # skip matrices beyond the largest layer of a 70B model (28672 x 8192)
+MAX_WEIGHTS = 240 * 1000 * 1000   # the grid skips matrices beyond the largest layer of a 70B model (28672 x 8192)
 # Layer shapes (OC, IC) of common decoder models that the grid does not hit: hidden/MLP sizes 2560, 3072, 3584, 5120, 6656,
 # 7168 with their fused QKV and gate+up projections (13B/14B/30B/32B LLaMA- and Qwen-shaped models, 7B Qwen2, Gemma, Phi-3,
 # OPT-30B).  Swept with `--pairs models`; off the grid the carry-over from neighbours costs 2 % on average, 15 % at worst.
@@ -53,7 +53,11 @@ MODEL_PAIRS = [(15360, 5120), (13824, 5120), (27648, 5120), (5120, 13824), (7168
                (3584, 3584), (4608, 3584), (18944, 3584), (37888, 3584), (3584, 18944),
                (3072, 3072), (9216, 3072), (16384, 3072), (24576, 3072), (49152, 3072), (3072, 24576),
                (2048, 16384), (2560, 2560), (7680, 2560), (2560, 9728), (9728, 2560), (19456, 2560),
-               (7168, 7168), (21504, 7168), (28672, 7168), (7168, 28672)]
+               (7168, 7168), (21504, 7168), (28672, 7168), (7168, 28672),
+               # the remaining shapes of the reference's run scripts (tests/python/run.sh:33-34, tests/cpp/run.sh:14-15): LLaMA-2-70B's fused
+               # gate+up projection and the OPT-66B / OPT-175B layers
+               (57344, 8192), (27648, 9216), (9216, 9216), (36864, 9216), (9216, 36864), (36864, 12288), (12288, 12288), (49152, 12288),
+               (12288, 49152)]
 
 
 def tile_rows(cfg):
@@ -155,7 +159,7 @@ def sweep(args):
     with open(args.out, "a" if args.append else "w") as f:
         for (OC, IC) in problems:
             if True:
-                if OC * IC > MAX_WEIGHTS:
+                if OC * IC > MAX_WEIGHTS and not args.pairs:
                     continue
                 for BS in Ns:
                     best = {}
