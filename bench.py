@@ -83,7 +83,7 @@ class Problem:
         from fp6_llm_amd import quant, synth
 
         self.E, self.M, self.OC, self.IC, self.BS = E, M, OC, IC, BS
-        self.splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC)
+        self.splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC, EXPONENT=E, MANTISSA=M)
         nbytes = fp6.native_bytes(E, M, OC, IC)
         self.nbuf = int(max(2, min(128, POOL_BYTES // nbytes)))
         # distinct buffers, distinct contents: uniform random codes (every bit pattern is a valid weight)

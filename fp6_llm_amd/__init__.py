@@ -27,13 +27,14 @@ from ._lib import Fp6miError  # noqa: F401
 
 # The native library is loaded on first use (every entry point raises ImportError while it is missing: there is no other
 # path), so that `python -m fp6_llm_amd.build` can import this package before anything is built.  The torch extension links
-# against it and is only tried once it is there.
+# against it and is only tried once it is there.  A library left over from an older source tree (a symbol missing) must not
+# stop the import either, or the build module could not be started to replace it: the first real call reports it.
 _ext = None
 if os.path.exists(_lib.LIB_PATH) and not os.environ.get("FP6MI_NO_TORCH_EXT"):
     try:
         _lib.lib()
         from . import _fp6mi_torch as _ext
-    except ImportError:   # not built (it needs torch's headers at build time): the ctypes path below does the same job
+    except (ImportError, OSError, AttributeError):   # extension not built, or a stale library: the ctypes path reports what is wrong
         _ext = None
 
 __all__ = [
@@ -63,10 +64,11 @@ def HeuristicFuntion_SplitK(M, N, Num_GPU_SMs):
     return 1
 
 
-def heuristic_splitk_mi355x(M, N, K, num_cus=MI355X_CUS):
+def heuristic_splitk_mi355x(M, N, K, num_cus=MI355X_CUS, EXPONENT=3, MANTISSA=2):
     """Split-K for this engine's kernels: K is already split across the wavefronts of a workgroup, so a split across
-    workgroups (second launch + FP32 workspace traffic) only pays when M/16 workgroups cannot occupy the chip."""
-    return _lib.lib().fp6mi_heuristic_splitk(M, N, K, num_cus)
+    workgroups (second launch + FP32 workspace traffic) only pays when M/16 workgroups cannot occupy the chip.  The answer
+    comes from the table measured for the format's bit width where the problem is near a measured one."""
+    return _lib.lib().fp6mi_heuristic_splitk_format(EXPONENT, MANTISSA, M, N, K, num_cus)
 
 
 # ----------------------------------------------------------------------------------------------------------------

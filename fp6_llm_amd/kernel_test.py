@@ -32,7 +32,7 @@ def run(OC, IC, BS, splitK=0, EXP=3, MAN=2, repeat=1000, warmup=10, seed=0, out=
     scale = (torch.rand(OC, generator=gen) + 0.5).half()
     act = (torch.rand(BS, IC, generator=gen) + 0.5).half()
     if splitK <= 0:
-        splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC)
+        splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC, EXPONENT=EXP, MANTISSA=MAN)
 
     dev = torch.device("cuda:0")
     packed = fp6.weight_prepacking_eXmY_cpu(EXP, MAN, raw).to(dev)

@@ -128,7 +128,7 @@ class FPxLinear(torch.nn.Module):
         if not sk:   # the heuristic's answer per batch size is remembered: the layer is called once per token
             sk = self._split_cache.get(x2.shape[0])
             if sk is None:
-                sk = self._split_cache[x2.shape[0]] = heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS)
+                sk = self._split_cache[x2.shape[0]] = heuristic_splitk_mi355x(self.out_features, x2.shape[0], self.in_features, MI355X_CUS, self.exponent, self.mantissa)
         y = linear_forward_native(self.exponent, self.mantissa, x2, self.weight_native, self.scales, self.out_features, sk, None, None, self.group_exps)
         if self.bias is not None:
             y = y + self.bias

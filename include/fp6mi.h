@@ -66,6 +66,8 @@ int    fp6mi_unpack_native(int E, int Mbits, void *raw, const void *native, size
  * HeuristicFuntion_SplitK, fp6_llm/__init__.py:13-23, whose model of one CTA per 512x64 outputs does not fit
  * this kernel).  Returns a value in [1, 64]. */
 int fp6mi_heuristic_splitk(size_t M, size_t N, size_t K, int num_cus);
+/* The same for a given weight format (the measured table is per bit width; the function above answers for FP6). */
+int fp6mi_heuristic_splitk_format(int E, int Mbits, size_t M, size_t N, size_t K, int num_cus);
 
 /* Bytes of the split-K workspace the GEMM entry points need: splitK*M*N floats (fp6_llm/csrc/fp6_linear.cuh:17),
  * 0 when splitK == 1. */

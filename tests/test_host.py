@@ -387,6 +387,16 @@ def test_module_construction_routes_agree():
         module.FPxLinear(100, 256)
 
 
+def test_split_heuristic_per_format():
+    L = _lib.lib()
+    for (M, N, K) in [(4096, 8, 4096), (8192, 32, 8192), (256, 8, 28672), (17920, 32, 6656), (1024, 300, 2048)]:
+        assert L.fp6mi_heuristic_splitk_format(3, 2, M, N, K, 256) == L.fp6mi_heuristic_splitk(M, N, K, 256)
+        assert L.fp6mi_heuristic_splitk_format(2, 3, M, N, K, 256) == L.fp6mi_heuristic_splitk(M, N, K, 256)   # same bytes, same table
+        for (E, Mb) in FORMATS:
+            s = fp6.heuristic_splitk_mi355x(M, N, K, EXPONENT=E, MANTISSA=Mb)
+            assert 1 <= s <= 64 and s <= (K + 255) // 256
+
+
 def test_fused_layers_are_the_concatenation():
     """Fusing layers over one input = quantizing the row-concatenated weight: native tiles are stored row tile after row tile."""
     from fp6_llm_amd import module
