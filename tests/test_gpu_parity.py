@@ -326,6 +326,18 @@ def test_command_line_harness(E, M):
     assert res["splitK"] == 2 and res["max_rel_err_vs_fp32"] <= 1e-2
 
 
+def test_command_line_harness_suites(monkeypatch):
+    """--suite walks a list of (OC, IC) shapes at the given batch sizes; the lists are the ones in the reference's run scripts."""
+    import io
+    from fp6_llm_amd import kernel_test
+    assert kernel_test.SUITES["llama2-70b"] == [(10240, 8192), (8192, 8192), (57344, 8192), (8192, 28672)]   # tests/python/run.sh:33-34
+    assert (13824, 5120) in kernel_test.SUITES["llama1-65b"] and (49152, 12288) in kernel_test.SUITES["opt"]
+    monkeypatch.setitem(kernel_test.SUITES, "tiny", [(256, 512), (512, 320)])
+    buf = io.StringIO()
+    rows = kernel_test.run_suite("tiny", [1, 20], 2, 1, 3, out=buf)
+    assert len(rows) == 4 and all(r["max_rel_err_vs_fp32"] <= 1e-2 for r in rows) and buf.getvalue().count("speed-up") == 4
+
+
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_random_shapes_through_the_automatic_launch_choice(E, M):
     """Forty seeded random problems per format -- rows in multiples of 256, columns in multiples of 64 (most of them not
