@@ -68,6 +68,16 @@ template <int FM> __device__ __forceinline__ WFrag<FM> load_wfrag(const uint8_t 
     return f;
 }
 
+// One of the two or three loads of load_wfrag, for a kernel that spreads them over its compute.
+template <int FM> __device__ __forceinline__ void load_wfrag_part(WFrag<FM> &f, const uint8_t *block, int lane, int part)
+{
+    const v4u *p = reinterpret_cast<const v4u *>(block) + lane;
+    if (part == 0) f.a = __builtin_nontemporal_load(p);
+    if (part == 1) f.b = __builtin_nontemporal_load(p + 64);
+    if constexpr (Fmt<FM>::bits == 6) { if (part == 2) f.c = __builtin_nontemporal_load(p + 128); }
+    if constexpr (Fmt<FM>::bits == 5) { if (part == 2) f.s = __builtin_nontemporal_load(reinterpret_cast<const v2u *>(block + 2048) + lane); }
+}
+
 // A operands (8 halfs = k 8q..8q+7 of this lane's row) of the eight MFMA steps of a block.
 // FP5: a quarter of the values (exact; the epilogue multiplies the sums by 4).  The other formats: exact values.
 template <int FM> struct AOps { v8h s[8]; };
@@ -421,6 +431,34 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
             }
         }
     };
+    // The same loads one at a time (i = 0 .. kLoads-1: weights first, then activation pieces).  The 256 x 128 tile spreads them
+    // over its MFMA steps instead of issuing them in one burst: measured 10-12 % faster for batches from 1024 up (the burst keeps
+    // a wavefront, which issues in order, from starting its MFMAs until the CU has accepted its last load); for the smaller
+    // tiles, with fewer MFMAs between two loads, spreading measured 0-8 % slower and they keep the burst.
+    constexpr bool kSpreadLoads = NT >= 8 && WR * WK >= 8;
+    constexpr int  kWParts = Fmt<FM>::bits == 4 ? 2 : 3, kWLoads = RT * kWParts, kLoads = kWLoads + kPerThread, kPerStep = (kLoads + 7) / 8;
+    auto load_one = [&](int i, uint32_t c0) {
+        if (i < kWLoads) {
+            const int      r = i / kWParts, part = i % kWParts;
+            const uint32_t u = c0 + wk;
+            if (u < u1) {
+                load_wfrag_part<FM>(wnxt[r], wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
+                if (part == 0) gnxt[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
+            }
+        } else if (i < kLoads) {
+            const int      j = i - kWLoads;
+            const uint32_t p = tid + NTHREADS * j;
+            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
+                if ((c0 + WK) * 256 <= K && c0 + WK <= u1) { // uniform
+                    xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
+                } else {
+                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
+                    const bool     ok = k < K && u < u1;
+                    xr[j] = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                }
+            }
+        }
+    };
     auto store_x = [&](int buf) {
 #pragma unroll
         for (int j = 0; j < kPerThread; j++)
@@ -435,7 +473,7 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         int buf = 0;
         for (uint32_t c0 = u0; c0 < u1; c0 += WK, buf ^= 1) {
             const bool more = c0 + WK < u1;
-            if (more) {
+            if (more && (!kSpreadLoads || c0 + wk >= u1)) { // (a wavefront without a K block in this chunk has no MFMAs to spread over)
                 load_x(c0 + WK);
                 load_w(wnxt, gnxt, c0 + WK);
             }
@@ -459,6 +497,12 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 #pragma unroll
                             for (int t = 0; t < NT; t++)
                                 acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h == 0 ? a0[r][s] : a1[r][s], b[t], acc[r][t], 0, 0, 0);
+                        if constexpr (kSpreadLoads) {
+                            if (more) {
+#pragma unroll
+                                for (int i = (4 * h + s) * kPerStep; i < (4 * h + s + 1) * kPerStep; i++) load_one(i, c0 + WK);
+                            }
+                        }
                     }
                 }
             }
