@@ -568,6 +568,27 @@ def test_device_groupwise_quantizer_matches_host_bits(E, M, dtype, OC, IC):
     assert torch.equal(native.cpu(), fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))))
 
 
+@pytest.mark.parametrize("E,M", [(3, 2), (2, 1)])
+def test_grouped_gemm_on_the_256x128_tile(E, M):
+    """A prefill-sized batch: the 256 x 128 tile, which spreads its loads (the group exponents among them) over the MFMA steps;
+    K = 1088 ends in a quarter-full K block.  Checked on a sample of rows against the definition."""
+    OC, IC, BS = 2048, 1088, 4096
+    shape = (ctypes.c_int * 5)()
+    assert _lib.lib().fp6mi_query_launch(E, M, OC, BS, IC, 1, shape) == 0 and tuple(shape) == (1, 8, 2, 8, 1)
+    codes, sc, ex = quant.quantize_groupwise(_grouped_weights(77, OC, IC), E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))).to(DEV)
+    gexp = fp6.pack_group_exps(torch.from_numpy(ex), OC, IC).to(DEV)
+    scd = torch.from_numpy(sc).to(DEV)
+    x = synth.activations(78, BS, IC)
+    xd = torch.from_numpy(x).to(DEV)
+    y = fp6.linear_forward_native(E, M, xd, native, scd, OC, 1, group_exps=gexp).cpu().numpy()
+    y_plain = fp6.linear_forward_native(E, M, xd, native, scd, OC, 1, group_exps=torch.full_like(gexp, 127))
+    assert torch.equal(y_plain, fp6.linear_forward_native(E, M, xd, native, scd, OC, 1))
+    rows = np.sort(np.random.default_rng(6).choice(OC, 192, replace=False))
+    wdq = oracle.dequant_grouped_from_definition(codes[rows], sc[rows], ex[rows], E, M)
+    check_close(y[:, rows], oracle.gemm_f64(wdq, x), "grouped, 256x128 tile")
+
+
 def test_grouped_module_forward_and_prefill_route():
     from fp6_llm_amd import module
     E, M, OC, IC = 2, 1, 512, 1024
