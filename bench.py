@@ -60,6 +60,7 @@ MEASURED_TRAFFIC_BYTES = {
     "fp6_4096x4096_bs8": 13239792,
     "fp6_8192x8192_bs8": 51576185,
     "fp5_8192x8192_bs8": 43183355,
+    "fp4_8192x8192_bs8": 34809973,
     "fp6_28672x8192_bs32": 182260903,
     "fp6_8192x8192_bs512": 125992391,
 }
