@@ -8,7 +8,7 @@ import torch
 
 from . import quant
 from . import (MI355X_CUS, group_exps_bytes, heuristic_splitk_mi355x, linear_forward_native, native_bytes, pack_group_exps, to_native,
-               weight_dequant_native_cuda, weight_prepacking_eXmY_cpu, weight_prepacking_native_cpu, weight_quantize_native_cuda)
+               weight_dequant_native_cuda, weight_prepacking_native_cpu, weight_quantize_native_cuda)
 
 _MAGIC = b"FP6MI\x00\x01\x00"   # name, NUL, layout version 1, reserved
 
