@@ -488,6 +488,29 @@ def test_config5_batch_sweep(E, M, BS):
     check_close(y[:, rows], oracle.gemm_f64(wdq, x), "8192x8192 BS=%d" % BS)
 
 
+def test_many_splits_reduce_in_split_order():
+    """Split counts that exercise every path of the reduction kernel (it keeps 8, 4, 2 or 1 partial sums in flight): the result
+    is the FP32 sum of the partial sums in split order, rounded once -- computed here from the workspace the GEMM left behind."""
+    E, M, OC, IC, BS = 3, 2, 256, 64 * 80, 9
+    raw, sc, x = synth.uniform_problem(808, OC, IC, BS, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    L = _lib.lib()
+    for splitK in (2, 3, 7, 8, 9, 11, 15, 16, 17, 20):
+        out = torch.empty((BS, OC), dtype=torch.float16, device=DEV)
+        ws = torch.zeros(splitK * BS * OC, dtype=torch.float32, device=DEV)
+        rc = L.fp6mi_linear_native(E, M, torch.cuda.current_stream().cuda_stream, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(),
+                                   OC, BS, IC, ws.data_ptr(), splitK)
+        assert rc == 0
+        torch.cuda.synchronize()
+        parts = ws.cpu().numpy().reshape(splitK, BS, OC)
+        acc = np.zeros((BS, OC), np.float32)
+        for s in range(splitK):
+            acc = acc + parts[s]                      # float32 additions in split order
+        assert (out.cpu().numpy().view(np.uint16) == acc.astype(np.float16).view(np.uint16)).all(), splitK
+        check_close(out.cpu().numpy(), ref, "splitK=%d" % splitK)
+
+
 def test_rows_of_very_different_magnitude():
     """The kernel multiplies the exact code values and scales the FP32 sum; the reference rounds every scaled weight to fp16
     first.  With rows whose outputs differ an order of magnitude that rounding alone moves the reference by 4.7e-3 of the global
