@@ -5,6 +5,7 @@ covers any shape; for the shapes of real models a measured table does better, th
 This tool measures every candidate shape on the GPU it runs on and writes that table:
 
     python -m fp6_llm_amd.tune sweep --format 6 --out fp6_llm_amd/tuning/fp6_mi355x.jsonl      # minutes of GPU time
+    python -m fp6_llm_amd.tune compact fp6_llm_amd/tuning/*.jsonl                               # after re-measuring with --append
     python -m fp6_llm_amd.tune emit fp6_llm_amd/tuning/*.jsonl                                  # -> csrc/fp6mi_tuning.inc
     python -m fp6_llm_amd.build
 
@@ -196,6 +197,19 @@ def emit(args):
     print("%d entries -> %s" % (len(rows), INC_PATH))
 
 
+def compact(args):
+    """Rewrites measurement files in place with one line per problem, the latest (re-measured shapes are appended by `sweep --append`)."""
+    for path in sorted(p for pat in args.files for p in glob.glob(pat)):
+        rows = {}
+        for line in open(path):
+            r = json.loads(line)
+            rows[(r["E"], r["M"], r["OC"], r["IC"], r["BS"])] = r
+        with open(path, "w") as f:
+            for key in sorted(rows):
+                f.write(json.dumps(rows[key]) + "\n")
+        print("%s: %d problems" % (path, len(rows)))
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__, formatter_class=argparse.RawDescriptionHelpFormatter)
     sub = ap.add_subparsers(dest="cmd", required=True)
@@ -214,6 +228,9 @@ def main(argv=None):
     e = sub.add_parser("emit")
     e.add_argument("files", nargs="+")
     e.set_defaults(fn=emit)
+    c = sub.add_parser("compact")
+    c.add_argument("files", nargs="+")
+    c.set_defaults(fn=compact)
     args = ap.parse_args(argv)
     args.fn(args)
 
