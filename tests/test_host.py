@@ -460,3 +460,33 @@ def test_tuner_candidates_and_table_emission(tmp_path, monkeypatch):
     tune.main(["emit", str(src)])
     lines = [l for l in (tmp_path / "out.inc").read_text().splitlines() if l.startswith("{")]
     assert lines == ["{6,2,16,8,{{0,1,1,1,8,160},{255,0,0,0,0,0},{0,1,2,1,4,200},{255,0,0,0,0,0}}},"]
+
+
+# ------------------------------------------------------------------------------------------------ randomized round trips
+def test_packers_round_trip_on_random_shapes_and_bits():
+    """Property check with hypothesis: for any supported format, any legal shape and any bit pattern, the reference layout and
+    the native layout both unpack to the raw tensor they were packed from, both routes to the native layout agree, and the
+    host prepacker equals the oracle's."""
+    from hypothesis import given, settings, strategies as st
+
+    @settings(max_examples=40, deadline=None)
+    @given(fmt=st.sampled_from(FORMATS), tiles=st.integers(1, 3), kblocks=st.integers(1, 9), seed=st.integers(0, 2 ** 31 - 1))
+    def check(fmt, tiles, kblocks, seed):
+        E, M = fmt
+        x = 1 + E + M
+        OC, IC = 64 * tiles, 64 * kblocks
+        raw = np.random.default_rng(seed).integers(0, 2 ** 32, size=(OC, IC // 32 * x), dtype=np.uint64).astype(np.uint32).view(np.int32)
+        L = _lib.lib()
+        packed, back = np.empty_like(raw), np.empty_like(raw)
+        assert L.fp6mi_prepack_ref(E, M, packed.ctypes.data, raw.ctypes.data, OC, IC) == 0
+        assert packed.tobytes() == oracle.prepack(raw, E, M).tobytes()
+        assert L.fp6mi_unpack_ref(E, M, back.ctypes.data, packed.ctypes.data, OC, IC) == 0 and (back == raw).all()
+        nat = np.empty(fp6.native_bytes(E, M, OC, IC), np.uint8)
+        nat2 = np.empty_like(nat)
+        assert L.fp6mi_prepack_native(E, M, nat.ctypes.data, raw.ctypes.data, OC, IC) == 0
+        assert L.fp6mi_relayout_ref_to_native(E, M, nat2.ctypes.data, packed.ctypes.data, OC, IC) == 0 and (nat == nat2).all()
+        back[:] = 0
+        assert L.fp6mi_unpack_native(E, M, back.ctypes.data, nat.ctypes.data, OC, IC) == 0 and (back == raw).all()
+
+    check()
+
