@@ -33,9 +33,11 @@ def max_value(E, M):
 
 
 def quantize_codes(values, E=3, M=2):
-    """values (any float array, already divided by the scale) -> uint8 codes, round-to-nearest, ties to the even code."""
+    """values (any float array, already divided by the scale) -> uint8 codes, round-to-nearest, ties to the even code.
+    +-Inf saturates to the largest magnitude, NaN becomes +0 (the device quantizer does the same)."""
     x = _check(E, M)
     v = np.asarray(values, dtype=np.float64)
+    v = np.where(np.isnan(v), 0.0, v)
     mags = magnitudes(E, M)
     a = np.minimum(np.abs(v), mags[-1])
     hi = np.clip(np.searchsorted(mags, a, side="left"), 0, len(mags) - 1)   # first magnitude >= a
@@ -47,11 +49,15 @@ def quantize_codes(values, E=3, M=2):
     return (sign << (x - 1)) | idx
 
 
+def _finite_abs(w):
+    return np.where(np.isfinite(w), np.abs(w), 0.0)
+
+
 def quantize_rowwise(weight, E=3, M=2):
     """weight [OC, IC] float -> (codes uint8 [OC, IC], scales float16 [OC]) with scale = absmax(row) / max_value,
     rounded to fp16 first so that codes are chosen against the scale that will actually be applied."""
     w = np.asarray(weight, dtype=np.float64)
-    absmax = np.abs(w).max(axis=1)
+    absmax = _finite_abs(w).max(axis=1)          # NaN and +-Inf do not set the scale
     scale = (absmax / max_value(E, M)).astype(np.float16)
     scale = np.where(scale == 0, np.float16(1.0), scale).astype(np.float16)
     return quantize_codes(w / scale.astype(np.float64)[:, None], E, M), scale
@@ -68,11 +74,11 @@ def quantize_groupwise(weight, E=3, M=2):
     w = np.asarray(weight, dtype=np.float64)
     OC, IC = w.shape
     top = max_value(E, M)
-    scale = (np.abs(w).max(axis=1) / top).astype(np.float16)
+    scale = (_finite_abs(w).max(axis=1) / top).astype(np.float16)
     scale = np.where(scale == 0, np.float16(1.0), scale).astype(np.float16)
     groups = (IC + GROUP - 1) // GROUP
     pad = np.zeros((OC, groups * GROUP))
-    pad[:, :IC] = np.abs(w)
+    pad[:, :IC] = _finite_abs(w)
     gmax = pad.reshape(OC, groups, GROUP).max(axis=2) / scale.astype(np.float64)[:, None]     # in units of the row scale
     with np.errstate(divide="ignore"):
         k = np.ceil(np.log2(gmax / top))                       # smallest k with gmax <= top * 2^k (checked below: log2 rounds)

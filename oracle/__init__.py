@@ -302,6 +302,93 @@ def dequant_grouped_from_definition(codes, scale, exps, E=3, M=2):
         return prod.astype(np.float16)
 
 
+# ---------------------------------------------------------------------------------------------- the quantizer, from its definition
+# The reference ships no rounding quantizer: its only cast truncates, throws out of range and is wired to no API
+# (fp6_llm/csrc/utils/weight_quant.h:9-105).  What the build's quantizers (numpy on the host, HIP on the device) must
+# produce is therefore fixed here by the definition alone, in exact arithmetic, sharing no code with either of them:
+#   scale[row] = fp16_rn(absmax(row) / max_value)   (absmax over the finite entries; 1.0 where that rounds to zero)
+#   code       = the representable magnitude nearest to |w| / scale[row], ties to the even code, clamped at max_value,
+#                with the sign of w;  NaN counts as +0, +-Inf as +-max_value.
+# PARITY UNPINNED against reference output (there is none to compare with); pinned by: quantize(value(code) * s) == code for
+# every code, ties between neighbours, monotonicity and the clamp (tests/test_oracle.py).
+
+
+def _fp16_rn_of_fraction(q):
+    """Round-to-nearest-even of a non-negative Fraction to binary16, returned as np.float16 (exact, no double rounding)."""
+    if q <= 0:
+        return np.float16(0.0)
+    e = q.numerator.bit_length() - q.denominator.bit_length()
+    if Fraction(2) ** e > q:
+        e -= 1
+    elif Fraction(2) ** (e + 1) <= q:
+        e += 1
+    ulp = Fraction(2) ** (max(e, -14) - 10)
+    n = q / ulp
+    fl = n.numerator // n.denominator
+    rem = n - fl
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and fl % 2 == 1):
+        fl += 1
+    v = fl * ulp
+    if v >= 65520:
+        return np.float16(np.inf)
+    return np.float16(float(v))     # exact: v is a binary16 value
+
+
+def _nearest_codes_exact(w, factor, E, M):
+    """codes for weights w (float64 holding fp16/bf16/fp32 values exactly) against per-element factors (float64 holding
+    fp16 scale times a power of two exactly).  |w| >= mid * factor is decided on exact products: a midpoint between two
+    neighbouring magnitudes has at most 7 significant bits and the factor 11, so mid * factor is exact in float64."""
+    x = bit_width(E, M)
+    mags = [abs(value_of_code(c, E, M)) for c in range(1 << (x - 1))]
+    a = np.abs(w)
+    idx = np.zeros(w.shape, dtype=np.int64)
+    for i in range(len(mags) - 1):
+        mid = float((mags[i] + mags[i + 1]) / 2)
+        bound = mid * factor
+        above = a > bound
+        tie = a == bound
+        # past the midpoint: at least i+1; exactly on it: the even one of i and i+1
+        idx = np.where(above | (tie & (i % 2 == 1)), np.maximum(idx, i + 1), idx)
+    idx = np.where(np.isnan(w), 0, idx)
+    sign = np.where(np.isnan(w), 0, np.signbit(w).astype(np.int64))
+    return ((sign << (x - 1)) | idx).astype(np.uint8)
+
+
+def quantize_from_definition(weight, E=3, M=2):
+    """weight [OC, IC] (float16 / float32 array; bf16 values passed as float32) -> (codes uint8 [OC, IC], scales float16 [OC])."""
+    x = bit_width(E, M)
+    w = np.asarray(weight, dtype=np.float64)
+    top = abs(value_of_code((1 << (x - 1)) - 1, E, M))
+    finite = np.where(np.isfinite(w), np.abs(w), 0.0)
+    scales = np.array([_fp16_rn_of_fraction(Fraction(float(m)) / top) for m in finite.max(axis=1)], dtype=np.float16)
+    scales = np.where(scales == 0, np.float16(1.0), scales).astype(np.float16)
+    return _nearest_codes_exact(w, np.broadcast_to(scales.astype(np.float64)[:, None], w.shape), E, M), scales
+
+
+def quantize_grouped_from_definition(weight, E=3, M=2):
+    """As quantize_from_definition, plus one exponent byte per (row, 128 columns): 127 + k with k the smallest integer in
+    [-15, 0] such that the group's largest finite |w| <= max_value * 2^k * scale[row] (decided on exact products); codes are
+    chosen against scale[row] * 2^k.  -> (codes, scales, exps uint8 [OC, ceil(IC/128)]).  PARITY UNPINNED like the
+    per-group scales themselves (no reference behaviour exists)."""
+    x = bit_width(E, M)
+    w = np.asarray(weight, dtype=np.float64)
+    OC, IC = w.shape
+    top = float(abs(value_of_code((1 << (x - 1)) - 1, E, M)))
+    finite = np.where(np.isfinite(w), np.abs(w), 0.0)
+    scales = np.array([_fp16_rn_of_fraction(Fraction(float(m)) / Fraction(top)) for m in finite.max(axis=1)], dtype=np.float16)
+    scales = np.where(scales == 0, np.float16(1.0), scales).astype(np.float16)
+    groups = (IC + 127) // 128
+    pad = np.zeros((OC, groups * 128))
+    pad[:, :IC] = finite
+    gmax = pad.reshape(OC, groups, 128).max(axis=2)
+    sc = scales.astype(np.float64)[:, None]
+    k = np.zeros((OC, groups), dtype=np.int64)
+    for cand in range(-1, -16, -1):      # top * 2^cand * scale is exact in float64 (4 + 11 significant bits)
+        k = np.where(gmax <= top * np.exp2(float(cand)) * sc, cand, k)
+    factor = np.repeat(np.exp2(k.astype(np.float64)), 128, axis=1)[:, :IC] * sc
+    return _nearest_codes_exact(w, factor, E, M), scales, (k + 127).astype(np.uint8)
+
+
 def gemm_f64(wdq, x):
     """float64 accumulation of the dequantized weights: the arbiter for GEMM tolerance checks. Returns float64 [N, OC]."""
     return np.asarray(x, dtype=np.float64) @ np.asarray(wdq, dtype=np.float64).T

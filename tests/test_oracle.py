@@ -26,7 +26,7 @@ ONES = {(2, 2): [272762913, 1107829124, 136414224, 562303042, 2215657992], (3, 2
 
 def _ones_raw(E, M, OC, IC):
     if (E, M) not in ONES:   # formats the reference's tests do not cover: the same tensor from the format definition
-        return quant.pack_raw(np.full((OC, IC), CODE_OF_ONE[(E, M)], np.uint8), E, M)
+        return oracle.codes_to_raw(np.full((OC, IC), CODE_OF_ONE[(E, M)], np.uint8), E, M).view(np.int32)
     words = np.array(ONES[(E, M)], dtype=np.uint32)
     reps = IC // (32 * len(words) // (1 + E + M))
     return np.tile(words, (OC, reps)).view(np.int32)
@@ -67,14 +67,14 @@ def test_golden_prepack_fixtures(golden_dir):
         # the fixture's input is what the generator produces from its seed (fixtures are reproducible)
         OC = z["raw"].shape[0]
         IC = z["raw"].shape[1] * 32 // (1 + E + M)
-        assert (quant.pack_raw(synth.uniform_codes(int(z["seed"]), OC, IC, E, M), E, M) == z["raw"]).all()
+        assert (oracle.codes_to_raw(synth.uniform_codes(int(z["seed"]), OC, IC, E, M), E, M).view(np.int32) == z["raw"]).all()
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_golden_hash_config1(golden_dir, E, M):
     name = "e%dm%d_256x1024_seed1001" % (E, M)
     ref = json.load(open(os.path.join(golden_dir, "prepack_hashes.json")))[name]
-    raw = quant.pack_raw(synth.uniform_codes(1001, 256, 1024, E, M), E, M)
+    raw = oracle.codes_to_raw(synth.uniform_codes(1001, 256, 1024, E, M), E, M).view(np.int32)
     assert hashlib.sha256(raw.tobytes()).hexdigest() == ref["raw_sha256"]
     assert hashlib.sha256(oracle.prepack(raw, E, M).tobytes()).hexdigest() == ref["packed_sha256"]
 
@@ -281,3 +281,81 @@ def test_gemm_against_float64_and_split_k():
         assert (np.abs(out - ref) / den).max() < 2e-3
     with pytest.raises(ValueError):
         oracle.gemm(wdq, x, 0)
+
+
+# ------------------------------------------------------------------------------------------------ the quantizer's definition
+def test_fp16_rounding_of_exact_fractions():
+    """oracle._fp16_rn_of_fraction against Python's binary16 packer on values that are exact doubles (so the packer sees the
+    true value and rounds once), including halfway cases, subnormals and the overflow threshold."""
+    rng = np.random.default_rng(77)
+    vals = [0.0, 2.0 ** -24, 2.0 ** -25, 3 * 2.0 ** -25, 2.0 ** -14, 65504.0, 65519.99, 1.0 + 2.0 ** -11, 1.0 + 3 * 2.0 ** -11,
+            (1 + 2.0 ** -10) * 2.0 ** -14, 6.1e-5, 0.333251953125]
+    vals += list(np.exp(rng.uniform(np.log(1e-8), np.log(6e4), 3000)))
+    vals += [float(np.float16(v)) + float(np.float16(v)) * 2.0 ** -11 for v in np.exp(rng.uniform(np.log(1e-4), np.log(3e4), 500))]   # near ties
+    for v in vals:
+        want = np.frombuffer(struct.pack("<e", v), dtype=np.float16)[0]
+        got = oracle._fp16_rn_of_fraction(Fraction(v))
+        assert got.view(np.uint16) == want.view(np.uint16), (v, got, want)
+    assert np.isinf(oracle._fp16_rn_of_fraction(Fraction(65520)))
+    # a value no double holds exactly: 1/3 rounds to 0x3555
+    assert oracle._fp16_rn_of_fraction(Fraction(1, 3)).view(np.uint16) == 0x3555
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_quantizer_definition_is_pinned(E, M):
+    """Nothing in the reference says which code a value rounds to (its cast truncates, utils/weight_quant.h:30-53), so the
+    definition in oracle.quantize_from_definition is pinned by what the mathematics fixes."""
+    x = 1 + E + M
+    half = 1 << (x - 1)
+    vals = np.array([float(oracle.value_of_code(c, E, M)) for c in range(1 << x)])
+    vals = np.copysign(np.abs(vals), np.where(np.arange(1 << x) >= half, -1.0, 1.0))
+    top = np.abs(vals).max()
+    for s in (1.0, 0.5, 0.0078125, 3.0, float(np.float16(0.00123)), float(np.float16(1.7)), 2.0 ** -20):
+        # every representable value times the scale maps back to its own code (the row holds the maximum, so scale == s)
+        codes, sc = oracle.quantize_from_definition((vals * s)[None, :], E, M)
+        assert float(sc[0]) == s, (s, sc)
+        assert (codes[0] == np.arange(1 << x)).all()
+        # midpoints between neighbours go to the even code; a hair to either side goes to that side
+        mags = np.abs(vals[:half])
+        mid = (mags[:-1] + mags[1:]) / 2
+        row = np.concatenate([[top], mid, mid * (1 + 2.0 ** -20), mid * (1 - 2.0 ** -20)]) * s
+        codes, sc = oracle.quantize_from_definition(row[None, :], E, M)
+        n = len(mid)
+        assert (codes[0, 1:1 + n] % 2 == 0).all() and (np.abs(codes[0, 1:1 + n].astype(int) - np.arange(n)) <= 1).all()
+        assert (codes[0, 1 + n:1 + 2 * n] == np.arange(1, n + 1)).all() and (codes[0, 1 + 2 * n:] == np.arange(n)).all()
+    # monotone, and never farther than half a step from the value
+    v = np.linspace(-top, top, 5001)
+    codes, sc = oracle.quantize_from_definition(v[None, :], E, M)
+    assert float(sc[0]) == 1.0
+    deq = vals[codes[0]]
+    assert (np.diff(deq) >= 0).all() and (np.abs(deq - v) <= np.diff(np.abs(vals[:half])).max() / 2).all()
+    # clamp, signs, zeros, non-finite entries
+    row = np.array([top, 5 * top, -7 * top, 0.0, -0.0, np.nan, np.inf, -np.inf])
+    codes, sc = oracle.quantize_from_definition(row[None, :], E, M)
+    assert float(sc[0]) == 5.0 or float(sc[0]) == 7.0     # absmax of the finite entries is 7 * top
+    assert codes[0].tolist()[2:] == [2 * half - 1, 0, half, 0, half - 1, 2 * half - 1]
+    z, sz = oracle.quantize_from_definition(np.zeros((2, 32)), E, M)
+    assert (z == 0).all() and (sz == 1).all()
+    # the scale is the correctly rounded quotient: absmax = top * s for an fp16 s gives s back, and one fp32 ulp more does too
+    s16 = np.float16(0.0123)
+    _, sc = oracle.quantize_from_definition(np.array([[top * float(s16) * (1 + 2.0 ** -23)]]), E, M)
+    assert sc[0] == s16
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_grouped_quantizer_definition(E, M):
+    """PARITY UNPINNED (no reference behaviour): the per-group exponent is the smallest of 112..127 that holds the group."""
+    x = 1 + E + M
+    top = float(abs(oracle.value_of_code((1 << (x - 1)) - 1, E, M)))
+    w = np.zeros((2, 384))
+    w[0, 0] = top                      # group 0 holds the row maximum: factor 1
+    w[0, 128] = top / 4                # exactly on a boundary: fits under 2^-2
+    w[0, 256] = top / 4 * (1 + 2.0 ** -20)   # a hair above it: needs 2^-1
+    w[1, 5] = 1.0
+    w[1, 300] = 2.0 ** -30             # far below: the smallest factor, 2^-15
+    codes, sc, ex = oracle.quantize_grouped_from_definition(w, E, M)
+    assert sc[0] == 1.0 and ex[0].tolist() == [127, 125, 126]
+    assert ex[1].tolist() == [127, 112, 112]
+    c_row, s_row = oracle.quantize_from_definition(w, E, M)
+    assert (s_row == sc).all() and (codes[:, :128] == c_row[:, :128]).all()
+    assert codes[0, 128] == (1 << (x - 1)) - 1      # against scale/4 the value top/4 is the largest code
