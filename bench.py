@@ -8,8 +8,11 @@ heuristic).  Weights are synthetic, already resident in HBM, and ROTATE through 
 256 MB last-level cache, so every step streams its weights from HBM like consecutive layers of a model would ("cold");
 --warm (and --sweep) add the same-buffer figure.  The K steps are captured once into a HIP graph and replayed inside
 the timed region, which removes the Python launch cost (~6 us/launch) from a ~5 us kernel.  The graph is first replayed
-untimed for ~60 ms (right after an idle spell the GPU runs 10-15 % slow), then five replays are timed one by one, each
-exactly K steps between two synchronizations, and the median is reported; the FP16 baseline is timed the same way.
+untimed for ~60 ms (right after an idle spell the GPU runs 10-15 % slow); then the K-step graph is replayed back to back, as
+many times as it takes to cover ~10 ms, between ONE pair of events, five times over, and the median is reported as time per
+step = event time / (replays x steps in the graph); a graph holds the K steps several times over when K is small -- a
+20-step graph would spread the 6-8 us between two replays over only 20 kernels of 5 us.  The FP16 baseline and the read-only floor are timed the same way.
+The default run also times one workload per benchmark configuration (`detail.configs`) beside an FP16 GEMM of its shape.
 
 Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth figure the reference's design is judged
 on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
@@ -54,13 +57,13 @@ HEADLINE = "fp6_4096x4096_bs8"
 
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
 # for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
-MEASURED_TRAFFIC_BYTES = {
-    "fp6_4096x4096_bs8": 13239792,
-    "fp6_8192x8192_bs8": 51576185,
-    "fp5_8192x8192_bs8": 43183355,
-    "fp4_8192x8192_bs8": 34809973,
-    "fp6_28672x8192_bs32": 182260903,
-    "fp6_8192x8192_bs512": 125992391,
+MEASURED_TRAFFIC_BYTES = {   # workload: bytes per launch, and fp6mi_version() of the library that was profiled
+    "fp6_4096x4096_bs8": {"bytes": 13239792, "lib_version": 110},
+    "fp6_8192x8192_bs8": {"bytes": 51576185, "lib_version": 110},
+    "fp5_8192x8192_bs8": {"bytes": 43183355, "lib_version": 110},
+    "fp4_8192x8192_bs8": {"bytes": 34809973, "lib_version": 110},
+    "fp6_28672x8192_bs32": {"bytes": 182260903, "lib_version": 110},
+    "fp6_8192x8192_bs512": {"bytes": 125992391, "lib_version": 110},
 }
 
 
@@ -90,9 +93,9 @@ class Problem:
         rows = min(OC, 1024)
         block = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(synth.uniform_codes(2001, rows, IC, E, M), E, M)))
         reps = OC // rows + (1 if OC % rows else 0)
-        base = block.repeat(reps)[: nbytes // 4].contiguous()
+        base = block.repeat(reps)[: nbytes // 4].contiguous().to(device)
         for i in range(self.nbuf):
-            self.weights.append(torch.roll(base, shifts=257 * i).to(device))
+            self.weights.append(torch.roll(base, shifts=257 * i) if i else base)
         self.scales = torch.from_numpy(synth.uniform_scales(2001, OC)).to(device)
         self.x = torch.from_numpy(synth.activations(2001, BS, IC)).to(device)
         self.out = torch.empty((BS, OC), dtype=torch.float16, device=device)
@@ -106,51 +109,67 @@ class Problem:
 
 
 CLOCK_WARMUP_MS = 60.0   # untimed graph replays before the timed ones: the first replays after an idle spell run 10-15 % slow
-TIMED_REPLAYS = 5        # each times exactly `steps` steps between two synchronizations; the median is reported
+TIMED_REGION_MS = 10.0   # one timed region = back-to-back replays of the K-step graph covering about this long
+TIMED_REGIONS = 5        # the median over this many regions is reported
 
 
 def _timed_replays(graph, steps):
-    """Replays the captured K-step graph untimed until the clocks have settled, then times TIMED_REPLAYS replays one by one.
-    Returns (median wall seconds, median HIP-event milliseconds) of one replay."""
+    """Replays the captured K-step graph untimed until the clocks have settled, then times TIMED_REGIONS regions of R
+    back-to-back replays each, R chosen so that a region lasts about TIMED_REGION_MS.
+    Returns (median wall seconds per step, median HIP-event microseconds per step, R)."""
     import torch
 
-    spent, n = 0.0, 0
-    while n < 2 or (spent < CLOCK_WARMUP_MS and n < 50):
+    spent, n, last = 0.0, 0, 0.0
+    while n < 2 or (spent < CLOCK_WARMUP_MS and n < 200):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        spent += e0.elapsed_time(e1)
+        last = e0.elapsed_time(e1)
+        spent += last
         n += 1
+    replays = int(max(1, min(20000, round(TIMED_REGION_MS / max(last, 1e-3)))))
     walls, evs = [], []
-    for _ in range(TIMED_REPLAYS):
+    for _ in range(TIMED_REGIONS):
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         e0.record()
-        graph.replay()
+        for _r in range(replays):
+            graph.replay()
         e1.record()
         torch.cuda.synchronize()
-        walls.append(time.perf_counter() - t0)
-        evs.append(e0.elapsed_time(e1))
-    return sorted(walls)[len(walls) // 2], sorted(evs)[len(evs) // 2]
+        walls.append((time.perf_counter() - t0) / (replays * steps))
+        evs.append(e0.elapsed_time(e1) * 1e3 / (replays * steps))
+    return sorted(walls)[len(walls) // 2], sorted(evs)[len(evs) // 2], replays
 
 
-def time_steps(prob, steps, warmup, cold):
-    """Returns (wall seconds between the two synchronizations, HIP-event milliseconds on the launch stream)."""
+MIN_GRAPH_STEPS = 240    # a captured graph holds the K steps this many times over if K is smaller: starting and ending a replay costs
+                         # 6-8 us on this stack, which a 20-step graph of 5 us kernels would book as 0.3-0.4 us per step
+
+
+def _capture_and_time(step, steps, warmup):
+    """`step(i)` enqueues step i on the current stream.  W eager warm-up steps, then the K steps (several times over when K is
+    small, see MIN_GRAPH_STEPS) captured into one graph and timed by _timed_replays; all figures are per step."""
     import torch
 
     stream = torch.cuda.Stream()
+    rounds = max(1, -(-MIN_GRAPH_STEPS // steps))
     with torch.cuda.stream(stream):
-        for i in range(warmup):
-            prob.step(i, cold)
+        for i in range(max(warmup, 1)):
+            step(i)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         with torch.cuda.graph(graph, stream=stream):
-            for i in range(steps):
-                prob.step(warmup + i, cold)
-        return _timed_replays(graph, steps)
+            for i in range(steps * rounds):
+                step(warmup + i)
+        return _timed_replays(graph, steps * rounds)
+
+
+def time_steps(prob, steps, warmup, cold):
+    """Returns (wall seconds per step, HIP-event microseconds per step on the launch stream, replays per timed region)."""
+    return _capture_and_time(lambda i: prob.step(i, cold), steps, warmup)
 
 
 def read_floor_us(prob, steps, warmup):
@@ -174,17 +193,7 @@ def read_floor_us(prob, steps, warmup):
         rc = lib.fp6mi_probe_stream_read(torch.cuda.current_stream().cuda_stream, w.data_ptr(), nbytes, sink.data_ptr())
         assert rc == 0, rc
 
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        for i in range(warmup):
-            step(i)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            for i in range(steps):
-                step(warmup + i)
-        _, ev_ms = _timed_replays(graph, steps)
-    return ev_ms * 1e3 / steps
+    return _capture_and_time(step, steps, warmup)[1]
 
 
 class _RocblasFp16:
@@ -218,35 +227,24 @@ class _RocblasFp16:
 def _time_fp16(fn, steps, warmup):
     import torch
 
-    for i in range(warmup):
-        fn(i)
-    torch.cuda.synchronize()
-    stream = torch.cuda.Stream()
-    with torch.cuda.stream(stream):
-        fn(0)
+    try:
+        return _capture_and_time(fn, steps, warmup)[1]
+    except RuntimeError:  # the BLAS library refused capture: time plain launches instead
         torch.cuda.synchronize()
-        try:
-            graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(graph, stream=stream):
-                for i in range(steps):
-                    fn(i)
-            _, ev_ms = _timed_replays(graph, steps)
-        except RuntimeError:  # the BLAS library refused capture: time plain launches instead
-            torch.cuda.synchronize()
-            for i in range(3 * steps):   # untimed, to settle the clocks
-                fn(i)
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            torch.cuda.synchronize()
-            e0.record()
-            for i in range(steps):
-                fn(i)
-            e1.record()
-            torch.cuda.synchronize()
-            ev_ms = e0.elapsed_time(e1)
-    return ev_ms * 1e3 / steps
+        for i in range(3 * steps):   # untimed, to settle the clocks
+            fn(i)
+        reps = max(steps, 200)
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        torch.cuda.synchronize()
+        e0.record()
+        for i in range(reps):
+            fn(i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) * 1e3 / reps
 
 
-def fp16_baseline_us(prob, steps, warmup):
+def fp16_baseline_us(prob, steps, warmup, with_rocblas=True):
     """FP16 GEMM of the same shape on the same GPU, weights rotating the same way: the counterpart of the reference's cuBLAS
     baseline (tests/python/kernel_test_fp6.py:45-62, tests/cpp/kernel_test_fpx.cu:80-103).  Two library paths are timed,
     torch F.linear (hipBLASLt) and rocblas_gemm_ex; returns (the faster one, {path: us})."""
@@ -259,6 +257,8 @@ def fp16_baseline_us(prob, steps, warmup):
     out = torch.empty(prob.BS, prob.OC, dtype=torch.float16, device=dev)
     res = {"torch_F_linear": _time_fp16(lambda i: torch.nn.functional.linear(prob.x, ws[i % nbuf]), steps, warmup)}
     try:
+        if not with_rocblas:
+            raise OSError("second library path not wanted")
         rb = _RocblasFp16()
         # same answer as F.linear before it is trusted as a baseline
         rb.linear(prob.x, ws[0], out, torch.cuda.current_stream().cuda_stream)
@@ -289,55 +289,86 @@ def fp16_system_blas_us(OC, IC, BS, steps):
     return float(m.group(1)) if res.returncode == 0 and m else None
 
 
-def cpu_baseline(E, M, OC, IC, BS, budget_s=15.0):
-    """The reference's CPU path on this host: weight_dequant_cpu (utils/weight_dequant.h:10-48, restated by the scalar C
-    oracle, one thread) followed by a torch CPU fp16 matmul (tests/python/kernel_test_fp6.py:48-58 on the CPU)."""
+def _cpu_model():
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def _best_median(fn, min_reps=3, budget_s=4.0):
+    ts = []
+    while len(ts) < min_reps or (sum(ts) < budget_s and len(ts) < 50):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[0], ts[len(ts) // 2], len(ts)
+
+
+def cpu_baseline(E, M, OC, IC, BS):
+    """The reference's CPU path on this host, each leg timed by itself (at least 3 repeats, best and median):
+      prepack  weight_matrix_prepacking      (utils/weight_prepacking.h:118-196)  -> this build's bit-exact fp6mi_prepack_ref (one thread per host cpu)
+      dequant  DeQuantMatrix_FPx_To_FP16     (utils/weight_dequant.h:10-48)       -> fp6mi_dequant (one thread per host cpu) and the scalar C oracle (1 thread)
+      matmul   torch CPU fp16 F.linear of the dequantized weights (tests/python/kernel_test_fp6.py:48-58, on the CPU)
+    `value` is the per-GEMM path the reference runs, dequantize + matmul, with the oracle's dequantizer (kind "port"), in
+    weight bytes per second; prepacking is ahead-of-time work and reported beside it."""
+    import numpy as np
     import torch
 
     import oracle
+    import fp6_llm_amd as fp6
     from fp6_llm_amd import quant, synth
 
     raw = quant.pack_raw(synth.uniform_codes(2001, OC, IC, E, M), E, M)
     sc = synth.uniform_scales(2001, OC)
     x = torch.from_numpy(synth.activations(2001, BS, IC))
-    reps, t_total, t_deq, t_mm = 0, 0.0, 0.0, 0.0
-    while reps < 3 or (t_total < budget_s and reps < 50):
-        t0 = time.perf_counter()
-        w = torch.from_numpy(oracle.dequant(raw, sc, E, M))
-        t1 = time.perf_counter()
-        torch.nn.functional.linear(x, w)
-        t2 = time.perf_counter()
-        reps += 1
-        t_deq += t1 - t0
-        t_mm += t2 - t1
-        t_total += t2 - t0
-    per = t_total / reps
+    raw_t, sc_t = torch.from_numpy(raw), torch.from_numpy(sc)
+    threads = int(torch.get_num_threads())
+    prepack = _best_median(lambda: fp6.weight_prepacking_eXmY_cpu(E, M, raw_t), budget_s=3.0)
+    deq_own = _best_median(lambda: fp6.weight_dequant_eXmY_cpu(E, M, raw_t, sc_t), budget_s=3.0)
+    deq_orc = _best_median(lambda: oracle.dequant(raw, sc, E, M), budget_s=5.0)
+    w = torch.from_numpy(oracle.dequant(raw, sc, E, M))
+    assert np.array_equal(fp6.weight_dequant_eXmY_cpu(E, M, raw_t, sc_t).numpy().view(np.uint16), w.numpy().view(np.uint16))
+    mm = _best_median(lambda: torch.nn.functional.linear(x, w), budget_s=3.0)
+    per = deq_orc[1] + mm[1]
+    ms = lambda t: round(t * 1e3, 3)
     return {
-        "value": round(weight_bytes(E, M, OC, IC) / per / 1e9, 4), "unit": "GB/s", "cores": int(torch.get_num_threads()), "kind": "port",
-        "sample": "%d x (oracle dequant %dx%d on 1 thread: %.1f ms + torch CPU fp16 F.linear BS=%d on %d threads: %.2f ms); host has %d cpus"
-                  % (reps, OC, IC, t_deq / reps * 1e3, BS, torch.get_num_threads(), t_mm / reps * 1e3, os.cpu_count()),
+        "value": round(weight_bytes(E, M, OC, IC) / per / 1e9, 4), "unit": "GB/s", "cores": threads, "kind": "port",
+        "sample": "FP%d %dx%d BS %d on '%s' (%d cpus, torch threads %d), median of >= 3 repeats per leg: oracle dequant (1 thread) %.1f ms + "
+                  "torch CPU fp16 F.linear (%d threads) %.2f ms per GEMM; ahead of time: fp6mi_prepack_ref (all host threads) %.1f ms; "
+                  "fp6mi_dequant (all host threads) %.1f ms"
+                  % (1 + E + M, OC, IC, BS, _cpu_model(), os.cpu_count(), threads, deq_orc[1] * 1e3, threads, mm[1] * 1e3, prepack[1] * 1e3, deq_own[1] * 1e3),
         "us_per_gemm": round(per * 1e6, 1),
+        "legs_ms": {"prepack_fp6mi_all_threads": {"best": ms(prepack[0]), "median": ms(prepack[1]), "repeats": prepack[2]},
+                    "dequant_fp6mi_all_threads": {"best": ms(deq_own[0]), "median": ms(deq_own[1]), "repeats": deq_own[2]},
+                    "dequant_oracle_1thread": {"best": ms(deq_orc[0]), "median": ms(deq_orc[1]), "repeats": deq_orc[2]},
+                    "matmul_torch_fp16": {"best": ms(mm[0]), "median": ms(mm[1]), "repeats": mm[2], "threads": threads}},
+        "cpu_model": _cpu_model(), "host_cpus": os.cpu_count(),
     }
 
 
-def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True, with_system_blas=True):
+def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True, with_system_blas=True, with_floor=True):
     E, M, OC, IC, BS = WORKLOADS[name]
     prob = Problem(E, M, OC, IC, BS, device)
-    wall_s, ev_ms = time_steps(prob, steps, warmup, cold=True)
-    us = ev_ms * 1e3 / steps
-    us_warm = time_steps(prob, steps, warmup, cold=False)[1] * 1e3 / steps if with_warm else float("nan")
+    wall_s, us, replays = time_steps(prob, steps, warmup, cold=True)
     wb = weight_bytes(E, M, OC, IC)
     flops = 2.0 * OC * IC * BS
     res = {
-        "workload": name, "us_per_gemm": round(us, 3), "us_per_gemm_wall": round(wall_s * 1e6 / steps, 3),
+        "workload": name, "us_per_gemm": round(us, 3), "us_per_gemm_wall": round(wall_s * 1e6, 3), "replays_per_timed_region": replays,
         "weight_GBps": round(wb / us / 1e3, 1), "tflops": round(flops / us / 1e6, 2),
         "hbm_frac": round(wb / us / 1e3 / HBM_PEAK_GBPS, 4), "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4),
         "splitK": prob.splitK, "weight_buffers": prob.nbuf, "weight_bytes": wb, "algorithmic_bytes": algorithmic_bytes(E, M, OC, IC, BS),
     }
     if with_warm:   # same weight buffer every step: served by the last-level cache when it fits
+        us_warm = time_steps(prob, steps, warmup, cold=False)[1]
         res["us_per_gemm_warm"] = round(us_warm, 3)
         res["weight_GBps_warm"] = round(wb / us_warm / 1e3, 1)
-    floor = read_floor_us(prob, steps, warmup)
+    floor = read_floor_us(prob, steps, warmup) if with_floor else None
     if floor is not None:
         res["read_floor_us"] = round(floor, 3)               # a kernel that only reads these weight buffers once
         res["read_floor_GBps"] = round(wb / floor / 1e3, 1)
@@ -346,33 +377,79 @@ def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True, wi
         del prob.weights[2:]
         import torch
         torch.cuda.empty_cache()
-        f16, paths = fp16_baseline_us(prob, min(steps, 200), min(warmup, 10))
+        f16, paths = fp16_baseline_us(prob, min(steps, 200), min(warmup, 10), with_rocblas=with_system_blas)
         if with_system_blas:
             del prob
             torch.cuda.empty_cache()
-            ext = fp16_system_blas_us(OC, IC, BS, min(steps, 500))
+            ext = fp16_system_blas_us(OC, IC, BS, 500)
             if ext is not None:
                 paths["system_rocblas_own_process"] = ext
                 f16 = min(f16, ext)
         res["fp16_gemm_us"] = round(f16, 3)             # the fastest of the FP16 library paths
         res["fp16_gemm_us_by_path"] = {k: round(v, 3) for k, v in paths.items()}
         res["speedup_vs_fp16"] = round(f16 / us, 3)
-    return res, wall_s
+    return res
+
+
+# One workload per benchmark configuration beyond the headline one, timed by the default run (`detail.configs`):
+# the MLP GEMMs of a 7B model at batch 32, the three GEMMs of a 70B layer at batch 32, and the 8192 x 8192 batch sweep's
+# ends and middle in both of the reference's formats.
+CONFIG_WORKLOADS = ["fp6_4096x4096_bs1", "fp6_4096x4096_bs16", "fp6_11008x4096_bs32", "fp6_4096x11008_bs32", "fp6_10240x8192_bs32",
+                    "fp6_28672x8192_bs32", "fp6_8192x28672_bs32", "fp6_8192x8192_bs1", "fp6_8192x8192_bs64", "fp6_8192x8192_bs512",
+                    "fp5_8192x8192_bs1", "fp5_8192x8192_bs64", "fp5_8192x8192_bs512"]
+
+
+def run_configs(device, budget_s):
+    """[{workload, us, hbm_frac | mfma_frac, fp16_us, speedup}] within a time budget (workloads that no longer fit are listed as skipped).
+    FP16 = torch F.linear (hipBLASLt) on fp16 weights of the same shape rotating the same way, same graph protocol."""
+    import torch
+
+    out, t0 = [], time.perf_counter()
+    for name in CONFIG_WORKLOADS:
+        if time.perf_counter() - t0 > budget_s:
+            out.append({"workload": name, "skipped": "time budget"})
+            continue
+        E, M, OC, IC, BS = WORKLOADS[name]
+        big = OC * IC > 64e6
+        r = run_workload(name, 40 if big else 100, 5, device, with_warm=False, with_system_blas=False, with_floor=False)
+        entry = {"workload": name, "us": r["us_per_gemm"], "splitK": r["splitK"], "weight_GBps": r["weight_GBps"], "tflops": r["tflops"]}
+        if BS >= 128:
+            entry["mfma_frac"] = r["mfma_frac"]
+        else:
+            entry["hbm_frac"] = r["hbm_frac"]
+        entry["fp16_us"] = r["fp16_gemm_us"]
+        entry["speedup"] = r["speedup_vs_fp16"]
+        out.append(entry)
+        torch.cuda.empty_cache()
+    return out
+
+
+def measured_traffic(workload):
+    """HBM bytes per launch from the committed profiler summary of this workload, or None when there is none or when it was
+    taken with another version of the library than the one loaded now (a changed kernel makes the figure stale)."""
+    import fp6_llm_amd._lib as _lib
+
+    rec = MEASURED_TRAFFIC_BYTES.get(workload)
+    if rec is None or rec["lib_version"] != _lib.lib().fp6mi_version():
+        return None
+    return rec["bytes"]
 
 
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=2000)
-    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default=HEADLINE, choices=sorted(WORKLOADS))
-    ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration")
+    ap.add_argument("--sweep", action="store_true", help="also run every benchmark configuration with all its legs")
     ap.add_argument("--sweep-out", default="bench_sweep.jsonl", help="where --sweep writes its JSON lines")
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the legs that run outside this process's GPU stream: the CPU path and the system-BLAS FP16 baseline (a child process)")
-    ap.add_argument("--warm", action="store_true", help="also time the workload with the same weight buffer every step (cache-resident weights)")
+    ap.add_argument("--no-configs", action="store_true", help="skip detail.configs (one workload per benchmark configuration)")
+    ap.add_argument("--configs-budget", type=float, default=75.0, help="seconds the default run may spend on detail.configs")
     ap.add_argument("--calibrate-copy", action="store_true",
-                    help="also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by")
+                    help="profiling aid: also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by; "
+                         "skips the FP16, CPU and per-configuration legs")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU (a linear layer shards by output rows without any collective); use --gpus 1")
@@ -380,6 +457,7 @@ def main():
     import torch
 
     import fp6_llm_amd  # noqa: F401  (raises if libfp6mi.so is missing: there is no fallback)
+    from fp6_llm_amd import _lib
 
     assert torch.cuda.is_available(), "bench.py needs the GPU"
     device = torch.device("cuda:0")
@@ -391,27 +469,32 @@ def main():
         for _ in range(10):
             dst.copy_(src)
         torch.cuda.synchronize()
-    res, wall_s = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy, with_warm=args.warm,
-                               with_system_blas=not args.no_cpu_baseline)
+    res = run_workload(args.workload, args.steps, args.warmup, device, with_fp16=not args.calibrate_copy, with_warm=not args.calibrate_copy,
+                       with_system_blas=not args.no_cpu_baseline)
     E, M, OC, IC, BS = WORKLOADS[args.workload]
+    res["lib_version"] = _lib.lib().fp6mi_version()
+    if not (args.no_configs or args.calibrate_copy):
+        res["configs"] = run_configs(device, args.configs_budget)
+    compute_bound = BS >= 128
     line = {
         "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(res["us_per_gemm"] / 1e3, 6),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "%s: FP%d_e%dm%d weights [%d,%d] x fp16 activations [%d,%d], weights rotating through %d distinct HBM buffers, splitK=%d"
                                % (args.workload, 1 + E + M, E, M, OC, IC, BS, IC, res["weight_buffers"], res["splitK"])},
-        "roofline": {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"], "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
-                     "bytes_per_launch": res["weight_bytes"], "kernel_us": res["us_per_gemm"]},
+        "roofline": ({"bound": "mfma", "achieved": res["tflops"], "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": res["mfma_frac"]} if compute_bound else
+                     {"bound": "hbm", "achieved": res["weight_GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": res["hbm_frac"]}),
         "detail": res,
     }
-    if not args.no_cpu_baseline:
+    line["roofline"].update({"traffic": measured_traffic(args.workload), "bytes_per_launch": res["weight_bytes"], "kernel_us": res["us_per_gemm"]})
+    if not (args.no_cpu_baseline or args.calibrate_copy):
         line["cpu_baseline"] = cpu_baseline(E, M, OC, IC, BS)
     if args.sweep:
         os.makedirs(os.path.dirname(os.path.abspath(args.sweep_out)), exist_ok=True)
         with open(args.sweep_out, "w") as f:
             for name in WORKLOADS:
                 big = WORKLOADS[name][2] * WORKLOADS[name][3] > 64e6
-                r, _ = run_workload(name, 100 if big else 300, 10, device)
+                r = run_workload(name, 40 if big else 100, 10, device)
                 f.write(json.dumps(r) + "\n")
                 f.flush()
                 print("%-22s %8.2f us  %7.0f GB/s (%.1f%% HBM)  %7.1f TFLOP/s  read-only %7.2f us  fp16 %8.2f us  x%.2f" % (
