@@ -7,6 +7,7 @@
 //   fp6mi_linear*      <- fpx_linear_kernel       fp6_llm/csrc/fp6_linear.cu:44-102
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <mutex>
 #include <type_traits>
 #include <unordered_map>
@@ -47,6 +48,21 @@ __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, con
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// Compute units of the current device, asked of the runtime once per device (the launch-shape rules and the measured table
+// are written for 256; another count takes the rules).
+int current_device_cus()
+{
+    static std::atomic<int> cus[64];
+    int                     dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
 
 // Rule for batches above 16 where no measured neighbour exists: score the six tile shapes that exhaustive sweeps showed to
 // cover every case (64x32 with four K wavefronts; 128x32 with one or two; 128x64 with two; 256x64; 256x128) and take the
@@ -244,7 +260,7 @@ inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, i
 int linear_native(const fp6mi::FormatOps &ops, hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, size_t M, size_t N, size_t K, float *ws,
                   int splitK, const LaunchCfg *forced)
 {
-    LaunchCfg c = forced ? *forced : pick_cfg(ops.bits, M, N, K, splitK, 256);
+    LaunchCfg c = forced ? *forced : pick_cfg(ops.bits, M, N, K, splitK, current_device_cus());
     if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
     int rc = ops.gemm(c, st, W, sc, gexp, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
@@ -272,12 +288,13 @@ const char *fp6mi_error_string(int code)
     case FP6MI_ERR_NULL: return "a required pointer is NULL";
     case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
     case FP6MI_ERR_SPLITK: return "splitK must be >= 1";
-    case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned";
+    case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned (scales: 8-byte)";
+    case FP6MI_ERR_CAPTURE: return "the stream is being captured and this call would have to allocate: convert the weights first (fp6mi_relayout_ref_to_native_gpu) or make the first call outside the capture";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fp6mi error";
     }
 }
 
-int fp6mi_version(void) { return 110; } // 110: e2m3 and e2m1, group exponents, per-format split heuristic
+int fp6mi_version(void) { return 120; } // 120: capture-safe fp6mi_linear, zero-filled activations beyond K
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
 int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }
@@ -339,14 +356,15 @@ static int heuristic_splitk(int xbits, size_t M, size_t N, size_t K, int num_cus
         return best_s;
     }
     const double cu_gbps = 60.0, hbm_gbps = 6000.0, launch_us = 3.0;
+    const double block_bytes = (double)fp6mi::native_block_bytes(xbits); // one 16-row x 256-column block of the format
     size_t       wgs = M / 16 ? M / 16 : 1;
     double       best = 1e30;
     int          best_s = 1;
     for (int s = 1; s <= 64 && (size_t)s <= units; s++) {
-        double per_wg_bytes = (double)((units + s - 1) / s) * 3072.0;
+        double per_wg_bytes = (double)((units + s - 1) / s) * block_bytes;
         double rounds = std::ceil((double)(wgs * (size_t)s) / (double)num_cus);
         double t_cu = rounds * per_wg_bytes / (cu_gbps * 1e3);
-        double t_hbm = (double)wgs * (double)units * 3072.0 / (hbm_gbps * 1e3);
+        double t_hbm = (double)wgs * (double)units * block_bytes / (hbm_gbps * 1e3);
         double t = launch_us + (t_cu > t_hbm ? t_cu : t_hbm);
         if (s > 1) t += launch_us + 2.0 * (double)s * (double)M * (double)N * 4.0 / (hbm_gbps * 1e3);
         if (t < best * 0.97) { best = t; best_s = s; }
@@ -364,6 +382,7 @@ static int check_gemm_args(int E, int Mb, const void *W, const void *sc, const v
     if (splitK < 1 || splitK > 65535) return FP6MI_ERR_SPLITK;
     if (splitK > 1 && !ws) return FP6MI_ERR_WORKSPACE;
     if (!aligned16(W) || !aligned16(B) || !aligned16(C) || (ws && !aligned16(ws))) return FP6MI_ERR_ALIGN;
+    if (reinterpret_cast<uintptr_t>(sc) & 7u) return FP6MI_ERR_ALIGN; // the tile kernel reads four row scales with one 8-byte load
     return FP6MI_OK;
 }
 
@@ -436,9 +455,17 @@ int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc,
             }
         }
         if (!native) {
+            // A twin has to be allocated and filled: not possible while the stream is being captured (the allocation would end
+            // the capture with an error, and a replay would not repeat it).
+            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+            if (hipError_t e = hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cap); e != hipSuccess) return (int)e;
+            if (cap != hipStreamCaptureStatusNone) return FP6MI_ERR_CAPTURE;
             size_t bytes = fp6mi::native_bytes(E, Mb, M, K);
             if (hipError_t e = hipMalloc(&native, bytes); e != hipSuccess) return (int)e;
-            rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K); // same stream: ordered before the GEMM
+            rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K);
+            // The twin becomes visible to other callers (and other streams) only once it is completely written: this
+            // one-time path waits for the relayout kernel before it publishes the pointer.
+            if (rc == 0) rc = (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
             if (rc != 0) {
                 (void)hipFree(native);
                 return rc;

@@ -203,7 +203,8 @@ __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t 
     }
     // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
-    // a multiple of 256) read position 0 of the row: the native layout holds zero weights there.
+    // a multiple of 256) count as zero activations against the zero weights the native layout holds there (0 x 0, whatever
+    // the row holds elsewhere: an infinite activation must not meet a padding weight).
     if (NT == 1 && xpack && (u + 1) * 256 <= K) { // uniform
         load_x_paired(st.x, xrow_packed + u * 256);
     } else
@@ -215,10 +216,14 @@ __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t 
     } else {
 #pragma unroll
         for (int s = 0; s < 8; s++) {
-            uint32_t k = u * 256 + 32 * s;
-            if (k + 8 * q >= K) k = 0;
+            uint32_t   k = u * 256 + 32 * s;
+            const bool beyond = k + 8 * q >= K; // such a piece is read at position 0 (a valid address) and replaced by zeros
+            if (beyond) k = 0;
 #pragma unroll
-            for (int t = 0; t < NT; t++) st.x[s][t] = *reinterpret_cast<const v8h *>(xrow[t] + k);
+            for (int t = 0; t < NT; t++) {
+                v4u v = *reinterpret_cast<const v4u *>(xrow[t] + k);
+                st.x[s][t] = __builtin_bit_cast(v8h, beyond ? (v4u){ 0u, 0u, 0u, 0u } : v);
+            }
         }
     }
     __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
@@ -404,8 +409,8 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     };
     // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
     // batch column (p/32) % TN, halfs 8*(p%32)..+7).  Row pointers and LDS offsets are fixed for the whole kernel.
-    // There is no zero fill: columns beyond N read the last real row (their outputs are never stored); positions beyond K or
-    // beyond the split read position 0 of the row (zero weights there, or a wavefront that does not compute).
+    // Columns beyond N read the last real row (their outputs are never stored); positions beyond K or beyond the split are
+    // read at position 0 of the row (a valid address) and staged as zeros (zero weights meet them, or no wavefront does).
     const half_t *xrow[kPerThread];
     uint32_t      xlds[kPerThread];
 #pragma unroll
@@ -426,7 +431,10 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
                 if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
                     const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
                     const bool     ok = k < K && u < u1;
-                    xr[j] = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                    {
+                        const v4u v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                        xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
+                    }
                 }
             }
         }
@@ -454,7 +462,10 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
                 } else {
                     const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
                     const bool     ok = k < K && u < u1;
-                    xr[j] = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                    {
+                        const v4u v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                        xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
+                    }
                 }
             }
         }
@@ -698,7 +709,7 @@ __global__ __launch_bounds__(256) void relayout_ref_to_native(uint8_t *__restric
 // Same arithmetic as the host quantizer of this package, so that both give identical bits:
 //   scale[row] = fp16_rn(absmax(row) / max_value) (1.0 where that rounds to zero), computed from a double quotient;
 //   code       = nearest representable magnitude to |w / scale| (a double quotient, clamped at max_value), ties to the even
-//                code, with the sign bit of w.
+//                code, with the sign bit of w.  NaN weights become +0, +-Inf saturates, and neither takes part in absmax.
 // (The reference's only quantizer truncates and is not wired to any API: fp6_llm/csrc/utils/weight_quant.h:9-105.)
 // ---------------------------------------------------------------------------------------------------------------
 template <typename T> __device__ __forceinline__ float to_float(T v);
@@ -718,6 +729,13 @@ __device__ __forceinline__ half_t half_rn_from_double(double q)
     return v >= 65520.0 ? (half_t)__builtin_inff() : (half_t)(float)v;
 }
 
+// |v| for finite v, 0 for NaN and +-Inf: neither sets a scale
+__device__ __forceinline__ float finite_abs(float v)
+{
+    const float a = fabsf(v);
+    return a <= 3.4028234663852886e38f ? a : 0.f;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void quant_row_scales(half_t *__restrict__ scales, const T *__restrict__ Wf, uint32_t M, uint32_t K,
                                                        double max_value)
@@ -729,7 +747,7 @@ __global__ __launch_bounds__(256) void quant_row_scales(half_t *__restrict__ sca
     float    amax = 0.f;
     for (uint32_t k = lane * 8; k < K; k += 512)
 #pragma unroll
-        for (int j = 0; j < 8; j++) amax = fmaxf(amax, fabsf(to_float<T>(p[k + j])));
+        for (int j = 0; j < 8; j++) amax = fmaxf(amax, finite_abs(to_float<T>(p[k + j])));
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) amax = fmaxf(amax, __shfl_xor(amax, off, 64));
     if (lane == 0) {
@@ -774,7 +792,7 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
             for (int s = 4 * h; s < 4 * h + 4; s++) {
                 const uint32_t k0 = U * 256 + 32 * s + 8 * q;
                 for (int j = 0; j < 8; j++)
-                    if (k0 + j < K) amax = fmaxf(amax, fabsf(to_float<T>(p[k0 + j])));
+                    if (k0 + j < K) amax = fmaxf(amax, finite_abs(to_float<T>(p[k0 + j])));
             }
             amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
             amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
@@ -796,8 +814,8 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
             if (k0 + j < K) {
                 float  w = to_float<T>(p[k0 + j]);
                 double a = fabs((double)w / f);
-                if (!(a <= max_value)) a = max_value; // clamps, and sends NaN to the maximum like a saturating cast
-                code = nearest_magnitude<FM>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (Fmt<FM>::bits - 1));
+                if (a > max_value) a = max_value; // clamps; +-Inf saturates
+                if (w == w) code = nearest_magnitude<FM>(a) | ((__builtin_bit_cast(uint32_t, w) >> 31) << (Fmt<FM>::bits - 1)); // NaN: +0
             }
             c[8 * s + j] = (uint8_t)code;
         }

@@ -236,6 +236,67 @@ def test_c_abi_drop_in_on_reference_layout(E, M):
     assert L.fp6mi_twin_clear() == 0
 
 
+def test_c_abi_drop_in_second_stream_and_capture():
+    """fp6mi_linear keeps a native twin per weight pointer.  A first call under stream capture must refuse (it would have to
+    allocate) instead of breaking the capture; once the twin exists, a call on another stream and a captured call both work."""
+    L = _lib.lib()
+    E, M, OC, IC, N = 3, 2, 512, 1024, 8
+    raw, sc, x = synth.uniform_problem(710, OC, IC, N, E, M)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    out = torch.zeros((N, OC), dtype=torch.float16, device=DEV)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    assert L.fp6mi_twin_clear() == 0
+    torch.cuda.synchronize()
+
+    def call(stream):
+        return L.fp6mi_linear(E, M, stream.cuda_stream, packed.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), OC, N, IC, None, 1)
+
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(sa):
+        with torch.cuda.graph(g, stream=sa):
+            rc_captured_first = call(sa)
+    assert rc_captured_first == -8, rc_captured_first      # FP6MI_ERR_CAPTURE; the capture itself stays intact
+    g.replay()                                              # an empty graph
+    torch.cuda.synchronize()
+    assert call(sa) == 0                                    # first real call: allocates and fills the twin on stream A
+    assert call(sb) == 0                                    # at once from stream B: the twin is complete by now
+    torch.cuda.synchronize()
+    check_close(out.cpu().numpy(), ref, "second stream")
+    out.zero_()
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(sb):
+        with torch.cuda.graph(g2, stream=sb):
+            assert call(sb) == 0                            # the twin exists: nothing to allocate, capture is fine
+    g2.replay()
+    torch.cuda.synchronize()
+    check_close(out.cpu().numpy(), ref, "captured call")
+    assert L.fp6mi_twin_clear() == 0
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("N", [8, 16, 40])
+def test_infinite_activation_next_to_padded_columns(E, M, N):
+    """K = 320 leaves 192 padding columns in the last 256-column block of the native layout.  An infinite activation in
+    column 0 must give infinite outputs of the right sign (where the weight of column 0 is not zero), not NaN from
+    infinity times a zero padding weight."""
+    OC, IC = 256, 320
+    raw, sc, x = synth.uniform_problem(720 + N, OC, IC, N, E, M)
+    x[:, 0] = np.float16(np.inf)
+    x[1::2, 0] = np.float16(-np.inf)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    wdq = oracle.dequant(raw, sc, E, M).astype(np.float64)
+    y = gemm_capi(E, M, native, scd, xd, OC).astype(np.float64)
+    with np.errstate(invalid="ignore"):
+        ref = x.astype(np.float64) @ wdq.T
+    w0 = wdq[:, 0]
+    nz = w0 != 0
+    assert nz.sum() > OC // 2
+    assert np.array_equal(np.isnan(y), np.isnan(ref)) and not np.isnan(y[:, nz]).any()
+    assert np.array_equal(y[:, nz], ref[:, nz])       # +-inf, exactly
+
+
 def test_torch_extension_and_ctypes_binding_agree(monkeypatch):
     """The per-call path exists twice over the same C ABI: the torch C++ extension (used when built) and ctypes."""
     assert fp6._ext is not None, "fp6_llm_amd/_fp6mi_torch.so is built by python -m fp6_llm_amd.build"
@@ -375,8 +436,19 @@ def _awkward_weights(seed, OC, IC, dtype):
     w[5, 0] = 28.0                                            # scale exactly 1.0: the row below sits on ties and exact values
     w[5, 1:65] = np.arange(64, dtype=np.float32) * 0.4375     # multiples of 7/16: many land midway between codes
     w[6, :] = -w[5, :]
+    w[7, 3] = np.nan                                          # NaN becomes +0, +-Inf saturates, neither sets the scale
+    w[7, 4] = np.inf
+    w[7, 5] = -np.inf
     t = torch.from_numpy(w).to(dtype)
     return t
+
+
+def _codes_of_native(native_dev, E, M, OC, IC):
+    """Codes [OC, IC] held by a native-layout device tensor (through fp6mi_unpack_native and the oracle's bit reader)."""
+    nat = native_dev.cpu().contiguous()
+    raw = np.zeros((OC, IC * (1 + E + M) // 8), dtype=np.uint8)
+    assert _lib.lib().fp6mi_unpack_native(E, M, raw.ctypes.data, nat.data_ptr(), OC, IC) == 0
+    return oracle.raw_to_codes(raw, E, M)
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
@@ -390,6 +462,10 @@ def test_device_quantizer_matches_host_bits(E, M, dtype, OC, IC):
     native_host = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M)))
     assert np.array_equal(scales.cpu().numpy().view(np.uint16), sc_host.view(np.uint16))
     assert torch.equal(native.cpu(), native_host)
+    # ... and the same as the definition evaluated in exact arithmetic by the oracle (which shares no code with either)
+    c_def, s_def = oracle.quantize_from_definition(w.float().numpy(), E, M)
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), s_def.view(np.uint16))
+    assert np.array_equal(_codes_of_native(native, E, M, OC, IC), c_def)
 
 
 def test_device_quantizer_rejects_bad_arguments():
@@ -589,6 +665,10 @@ def test_device_groupwise_quantizer_matches_host_bits(E, M, dtype, OC, IC):
     assert np.array_equal(scales.cpu().numpy().view(np.uint16), sc_host.view(np.uint16))
     assert torch.equal(gexp.cpu(), fp6.pack_group_exps(torch.from_numpy(ex_host), OC, IC))
     assert torch.equal(native.cpu(), fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))))
+    c_def, s_def, e_def = oracle.quantize_grouped_from_definition(w.float().numpy(), E, M)
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), s_def.view(np.uint16))
+    assert torch.equal(gexp.cpu(), fp6.pack_group_exps(torch.from_numpy(e_def), OC, IC))
+    assert np.array_equal(_codes_of_native(native, E, M, OC, IC), c_def)
 
 
 @pytest.mark.parametrize("E,M", [(3, 2), (2, 1)])

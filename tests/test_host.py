@@ -165,7 +165,8 @@ def test_error_codes_instead_of_aborts():
     assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 1, 64, None, 0) == -5
     assert L.fp6mi_linear_native(3, 2, None, None, p, p, p, 256, 1, 64, None, 1) == -3
     assert L.fp6mi_linear_native(3, 2, None, p + 4, p, p, p, 256, 1, 64, None, 1) == -6  # alignment
-    for code in (-1, -2, -3, -4, -5, -6):
+    assert L.fp6mi_linear_native(3, 2, None, p, p + 2, p, p, 256, 1, 64, None, 1) == -6  # scales: 8-byte alignment
+    for code in (-1, -2, -3, -4, -5, -6, -8):
         assert len(L.fp6mi_error_string(code)) > 8
     assert L.fp6mi_workspace_bytes(256, 8, 1) == 0 and L.fp6mi_workspace_bytes(256, 8, 3) == 3 * 256 * 8 * 4
 
@@ -274,6 +275,43 @@ def test_quantizer(E, M):
     assert np.abs(deq - w).max() <= np.abs(w).max() / mags[-1] * np.diff(mags).max() * 0.51
     raw = quant.pack_raw(codes, E, M)
     assert (quant.unpack_raw(raw, E, M) == codes).all() and (oracle.unpack_codes(raw, E, M) == codes).all()
+
+
+def _awkward_weights(seed, OC, IC):
+    """Gaussian weights with what a quantizer gets wrong: zero rows, a row whose scale is an fp16 subnormal, a huge row,
+    negative zeros, exact ties of the scaled grid, and NaN / +-Inf entries."""
+    w = synth.normal(seed, (OC, IC)).astype(np.float32)
+    w[1, :] = 0.0
+    w[2, :] *= 1e-7
+    w[3, :] *= 3000.0
+    w[4, ::3] = -0.0
+    w[5, :] = 0.0
+    w[5, 0] = 28.0
+    w[5, 1:65] = np.arange(64, dtype=np.float32) * 0.4375
+    w[6, :] = -w[5, :]
+    w[7, 3] = np.nan
+    w[7, 4] = np.inf
+    w[7, 5] = -np.inf
+    return w
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("dtype", [np.float16, np.float32])
+def test_host_quantizer_equals_the_exact_definition(E, M, dtype):
+    """quant.quantize_rowwise / quantize_groupwise (float64 quotients, searchsorted) against the oracle's definition in exact
+    arithmetic: same scales, same codes, same group exponents."""
+    with np.errstate(over="ignore"):
+        w = _awkward_weights(61, 64, 320).astype(dtype)
+    codes, sc = quant.quantize_rowwise(w, E, M)
+    c0, s0 = oracle.quantize_from_definition(w, E, M)
+    assert np.array_equal(sc.view(np.uint16), s0.view(np.uint16)) and np.array_equal(codes, c0)
+    spread = np.exp(np.random.default_rng(5).normal(0, 2.0, (64, 3))).repeat(128, axis=1)[:, :320]
+    spread[:8] = 1.0
+    with np.errstate(over="ignore", invalid="ignore"):
+        wg = (w.astype(np.float64) * spread).astype(dtype)
+    codes, sc, ex = quant.quantize_groupwise(wg, E, M)
+    c0, s0, e0 = oracle.quantize_grouped_from_definition(wg, E, M)
+    assert np.array_equal(sc.view(np.uint16), s0.view(np.uint16)) and np.array_equal(ex, e0) and np.array_equal(codes, c0)
 
 
 def test_native_weight_file_round_trip(tmp_path):
