@@ -289,12 +289,13 @@ const char *fp6mi_error_string(int code)
     case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
     case FP6MI_ERR_SPLITK: return "splitK must be >= 1";
     case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned (scales: 8-byte)";
+    case FP6MI_ERR_TOO_LARGE: return "splitK*M*N floats exceed the library's static workspace (fp6mi_static_workspace_bytes)";
     case FP6MI_ERR_CAPTURE: return "the stream is being captured and this call would have to allocate: convert the weights first (fp6mi_relayout_ref_to_native_gpu) or make the first call outside the capture";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fp6mi error";
     }
 }
 
-int fp6mi_version(void) { return 120; } // 120: capture-safe fp6mi_linear, zero-filled activations beyond K
+int fp6mi_version(void) { return 120; } // 120: allocation-free entry point over a static workspace, capture-safe fp6mi_linear
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
 int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }
@@ -425,6 +426,55 @@ int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, 
     LaunchCfg c = pick_cfg(1 + E + Mb, M, N, K, splitK, 256);
     shape[0] = c.kind, shape[1] = c.nt, shape[2] = c.rt, shape[3] = c.wr, shape[4] = c.wk;
     return FP6MI_OK;
+}
+
+// ---- allocation-free variant of fp6mi_linear_native: the split-K workspace is a static device array of the library ----
+namespace {
+constexpr size_t kStaticWsFloats = (size_t)8 << 20; // 32 MiB per GPU, held from the first use of the library on that GPU until the process ends
+__device__ __align__(256) float g_static_ws[kStaticWsFloats];
+
+// Device address of g_static_ws on the current device (every GPU holds its own copy of the array at its own address); asked
+// of the runtime once per device.  The array's name is only a host-side handle: kernels get this pointer as an argument.
+int static_ws_ptr(float **out)
+{
+    static std::mutex mu;
+    static float     *ptrs[64];
+    int               dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= 64) return FP6MI_ERR_SHAPE;
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void *p = nullptr;
+        if (hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_ws)); e != hipSuccess) return (int)e;
+        ptrs[dev] = static_cast<float *>(p);
+    }
+    *out = ptrs[dev];
+    return FP6MI_OK;
+}
+} // namespace
+
+size_t fp6mi_static_workspace_bytes(void) { return kStaticWsFloats * sizeof(float); }
+
+int fp6mi_init(void)
+{
+    float *p = nullptr;
+    (void)current_device_cus();
+    return static_ws_ptr(&p);
+}
+
+int fp6mi_linear_native_static(int E, int Mb, void *stream, const void *W, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
+                               int splitK)
+{
+    float *ws = nullptr;
+    if (splitK > 1) {
+        // checked before the multiplication can overflow: M, N <= 2^31 and splitK <= 65535 are enforced by check_gemm_args below
+        if (M > 0x7fffffffu || N > 0x7fffffffu || splitK > 65535) return FP6MI_ERR_SHAPE;
+        if ((size_t)splitK * M > kStaticWsFloats || (size_t)splitK * M * N > kStaticWsFloats) return FP6MI_ERR_TOO_LARGE;
+        if (int rc = static_ws_ptr(&ws); rc != FP6MI_OK) return rc;
+    }
+    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    return linear_native(*fp6mi::ops_for(E, Mb), static_cast<hipStream_t>(stream), W, sc, nullptr, B, C, M, N, K, ws, splitK, nullptr);
 }
 
 // ---- drop-in entry on REFERENCE-layout weights: native twins are made on first sight of a weight pointer and kept ----

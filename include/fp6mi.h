@@ -37,6 +37,7 @@ extern "C" {
 #define FP6MI_ERR_WORKSPACE (-4) /* splitK > 1 without a workspace          */
 #define FP6MI_ERR_SPLITK (-5)    /* splitK < 1                              */
 #define FP6MI_ERR_ALIGN (-6)     /* a device pointer is not 16-byte aligned (scales: 8-byte) */
+#define FP6MI_ERR_TOO_LARGE (-7) /* the problem exceeds the static workspace of fp6mi_linear_native_static */
 #define FP6MI_ERR_CAPTURE (-8)   /* the call would have to allocate while its stream is being captured */
 
 const char *fp6mi_error_string(int code);
@@ -83,6 +84,20 @@ size_t fp6mi_workspace_bytes(size_t M, size_t N, int splitK);
  * (role of include/kernel_reduction.cuh:28-47) produces C.  M % 256 == 0, K % 64 == 0, N >= 1. */
 int fp6mi_linear_native(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
                         const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK);
+
+/* Allocation-free variant of fp6mi_linear_native.  It has no counterpart in the reference (whose callers bring the
+ * workspace, fp6_llm/csrc/fp6_linear.cuh:17); it is for callers that can neither allocate nor keep a workspace: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same kernels and results as
+ * fp6mi_linear_native; the split-K partial sums go to a static device array of the library,
+ * fp6mi_static_workspace_bytes() bytes (32 MiB) per GPU, instead of a caller workspace.  It calls no hipMalloc/hipFree.
+ * splitK * M * N floats beyond that size return FP6MI_ERR_TOO_LARGE.  All calls on one GPU share the array: calls with
+ * splitK > 1 that overlap in time on one GPU (different streams) race; calls on one stream are ordered.
+ * fp6mi_init() looks the array's device address up for the current device ahead of time (the first call on a device does
+ * it otherwise); call it once per device outside any stream capture. */
+int    fp6mi_linear_native_static(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
+                                  const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, int splitK);
+size_t fp6mi_static_workspace_bytes(void);
+int    fp6mi_init(void);
 
 /* Drop-in for fp_eXmY_linear_kernel / fp6_linear_kernel (fp6_llm/csrc/fp6_linear.cuh:8-32): W is the REFERENCE
  * prepacked layout on the device, exactly what a caller of the reference already holds.  On the first call with a
