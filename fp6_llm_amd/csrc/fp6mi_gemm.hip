@@ -191,10 +191,14 @@ template <int FM, int NT, int RT> struct Stage {
     v8h       x[8][NT];
 };
 
-template <int FM, bool GS, int NT, int RT>
+// How the activations of a K block are fetched: kXPaired (batches up to 8, block wholly inside K: two MFMA steps per load),
+// kXFull (block wholly inside K) or kXTail (the last block of a K that is not a multiple of 256).  The kernel chooses
+// outside its K loop: a choice made per block inside the loop cost 0.2 us of a 4.9 us launch at 4096 x 4096.
+enum XMode { kXPaired, kXFull, kXTail };
+
+template <int FM, bool GS, int NT, int RT, XMode MODE>
 __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, const uint8_t *ggroup, uint32_t units,
-                                           uint32_t u, int lane, const half_t *const (&xrow)[NT], int q, uint32_t K, bool xpack,
-                                           const half_t *xrow_packed)
+                                           uint32_t u, int lane, const half_t *const (&xrow)[NT], int q, uint32_t K, const half_t *xrow_packed)
 {
 #pragma unroll
     for (int r = 0; r < RT; r++) {
@@ -205,10 +209,10 @@ __device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t 
     // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
     // a multiple of 256) count as zero activations against the zero weights the native layout holds there (0 x 0, whatever
     // the row holds elsewhere: an infinite activation must not meet a padding weight).
-    if (NT == 1 && xpack && (u + 1) * 256 <= K) { // uniform
+    if constexpr (MODE == kXPaired) {
+        static_assert(NT == 1, "paired activation loads serve one column tile");
         load_x_paired(st.x, xrow_packed + u * 256);
-    } else
-    if ((u + 1) * 256 <= K) { // uniform: whole block inside K, one base address and immediate offsets
+    } else if constexpr (MODE == kXFull) { // one base address and immediate offsets
 #pragma unroll
         for (int s = 0; s < 8; s++)
 #pragma unroll
@@ -243,7 +247,7 @@ __device__ __forceinline__ void consume_stage(const Stage<FM, NT, RT> &st, v4f (
     }
 }
 
-template <int FM, bool GS, int NT, int RT, int WAVES>
+template <int FM, bool GS, int NT, int RT, int WAVES, bool SPLIT>
 __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
                                                             const uint8_t *__restrict__ gexp, const half_t *__restrict__ X, half_t *__restrict__ C,
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
@@ -251,13 +255,21 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 {
     __shared__ float red[WAVES][RT * NT][256];
 
-    const int      lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    // every kernel argument is fetched by one batch of scalar loads at the top (left alone, the compiler fetches them in
+    // three batches, each a round trip to memory, as the code reaches their first use)
+    asm volatile("" ::"s"(W), "s"(scales), "s"(gexp), "s"(X), "s"(C), "s"(ws), "s"(M), "s"(N), "s"(K), "s"(units), "s"(splitK));
+    // the wavefront's index as a scalar: the K-block loop, its bounds and its branches then run on the scalar unit
+    const int      lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int      col = lane & 15, q = lane >> 4;
     const uint32_t R0 = blockIdx.x * RT, split = blockIdx.y, nbase = blockIdx.z * (16 * NT);
 
-    const uint32_t avg = units / splitK, extra = units % splitK;
-    const uint32_t u0 = split * avg + (split < extra ? split : extra);
-    const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
+    // SPLIT = false is the launch with splitK == 1: its range is the whole of K and its epilogue writes fp16
+    uint32_t u0 = 0, u1 = units;
+    if constexpr (SPLIT) {
+        const uint32_t avg = units / splitK, extra = units % splitK;
+        u0 = split * avg + (split < extra ? split : extra);
+        u1 = u0 + avg + (split < extra ? 1u : 0u);
+    }
 
     const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
@@ -276,7 +288,6 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         xrow[t]    = X + (size_t)(n < N ? n : N - 1) * K + 8 * q;
     }
     // batches up to 8: two MFMA steps per activation load (see load_x_paired)
-    const bool    xpack = NT == 1 && N <= 8;
     const int     prow = col & 7, pstep = col >> 3;
     const half_t *xrow_packed = X + (size_t)((uint32_t)prow < N ? prow : N - 1) * K + 8 * q + 32 * pstep;
 
@@ -294,11 +305,21 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     // the same activation lines of the same L2 channel at the same moment
     // One K block at a time and no register double-buffering: the other wavefronts of the workgroup keep the memory system
     // busy while this one converts, and a second stage in registers measured slower at every size.
-    for (uint32_t u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES); u < u1; u += WAVES) {
-        Stage<FM, NT, RT> cur;
-        load_stage<FM, GS, NT, RT>(cur, wgroup, tile_stride, ggroup, units, u, lane, xrow, q, K, xpack, xrow_packed);
-        consume_stage<FM, GS, NT, RT>(cur, acc);
+    const uint32_t ufull = K / 256 < u1 ? K / 256 : u1; // the blocks before this one lie wholly inside K
+    uint32_t       u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES);
+    auto           run = [&](auto mode, uint32_t end) {
+        for (; u < end; u += WAVES) {
+            Stage<FM, NT, RT> cur;
+            load_stage<FM, GS, NT, RT, decltype(mode)::value>(cur, wgroup, tile_stride, ggroup, units, u, lane, xrow, q, K, xrow_packed);
+            consume_stage<FM, GS, NT, RT>(cur, acc);
+        }
+    };
+    if (NT == 1 && N <= 8) {
+        if constexpr (NT == 1) run(std::integral_constant<XMode, kXPaired>{}, ufull);
+    } else {
+        run(std::integral_constant<XMode, kXFull>{}, ufull);
     }
+    run(std::integral_constant<XMode, kXTail>{}, u1); // at most one block, and only when K is not a multiple of 256
 
     // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
 #pragma unroll
@@ -320,7 +341,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
         if (ng < N) {
             float v = sum * ((float)my_scale[j] * Fmt<FM>::post_scale);
-            if (splitK == 1)
+            if constexpr (!SPLIT)
                 C[(size_t)ng * M + mg] = (half_t)v;
             else
                 ws[((size_t)split * N + ng) * M + mg] = v;
@@ -361,7 +382,8 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     constexpr int  kPieces = WK * TN * 32, kPerThread = (kPieces + NTHREADS - 1) / NTHREADS;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    asm volatile("" ::"s"(W), "s"(scales), "s"(gexp), "s"(X), "s"(C), "s"(ws), "s"(M), "s"(N), "s"(K), "s"(units), "s"(splitK), "s"(nblocks)); // one batch of argument loads
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6); // a scalar, like all that follows from it
     const int wr = wave % WR, wk = wave / WR;
     const int col = lane & 15, q = lane >> 4;
 
@@ -372,9 +394,12 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     const uint32_t nb = id % nblocks, rest = id / nblocks, split = rest % splitK, mb = rest / splitK;
     const uint32_t nbase = nb * TN, R0 = (mb * WR + wr) * RT; // first row tile of this wavefront
 
-    const uint32_t avg = units / splitK, extra = units % splitK;
-    const uint32_t u0 = split * avg + (split < extra ? split : extra);
-    const uint32_t u1 = u0 + avg + (split < extra ? 1u : 0u);
+    uint32_t u0 = 0, u1 = units;
+    if (splitK > 1) {
+        const uint32_t avg = units / splitK, extra = units % splitK;
+        u0 = split * avg + (split < extra ? split : extra);
+        u1 = u0 + avg + (split < extra ? 1u : 0u);
+    }
 
     const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
@@ -830,9 +855,15 @@ int launch_stream(hipStream_t st, const void *W, const void *sc, const void *gex
 {
     uint32_t units = (uint32_t)((K + 255) / 256);
     dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    hipLaunchKernelGGL((gemm_stream<FM, GS, NT, RT, WAVES>), grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W),
-                       static_cast<const half_t *>(sc), static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws,
-                       (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK);
+    auto     go = [&](auto kernel) {
+        hipLaunchKernelGGL(kernel, grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc),
+                           static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N,
+                           (uint32_t)K, units, (uint32_t)splitK);
+    };
+    if (splitK > 1)
+        go(gemm_stream<FM, GS, NT, RT, WAVES, true>);
+    else
+        go(gemm_stream<FM, GS, NT, RT, WAVES, false>);
     return (int)hipGetLastError();
 }
 
