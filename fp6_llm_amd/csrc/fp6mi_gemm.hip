@@ -165,86 +165,28 @@ template <int FM, bool GS> __device__ __forceinline__ void convert(const WFrag<F
 //   grid  = (M/(16*RT) row groups, splitK, ceil(N / (16*NT)))      block = WAVES wavefronts
 // A workgroup owns 16*RT output rows and 16*NT batch columns over the K blocks of its split; its wavefronts take the
 // blocks round-robin (K is split inside the workgroup), each streaming its weights HBM -> VGPR and its slice of the
-// activations L2 -> VGPR directly in MFMA B-operand order (reused for the RT row tiles); the partial accumulators are
-// summed through LDS.
+// activations L2 -> VGPR -> LDS -> VGPR (reused for the RT row tiles); the partial accumulators are summed through LDS.
+//
+// Why the activations take the detour through LDS.  The MFMA wants lane (col, q) to hold 16 bytes of batch row `col`, so a
+// load in operand order makes the 16 lanes of every quarter-wavefront touch 16 different 128-byte lines, 16 bytes of each.
+// The vector memory pipeline looks up one line per cycle: measured on the MI355X with nothing else in the kernel, the
+// operand-order loads of a 4096-wide K for batch 16 on all 256 CUs take 3.1 us, the same bytes loaded as whole rows
+// (32 consecutive lanes = 512 consecutive bytes) 0.9 us; batch 8 with two MFMA steps per load 1.4 us against 0.25 us.
+// So every wavefront loads its slice as whole rows, writes it to an LDS area of its own (no barrier: nobody else reads it)
+// and reads it back in operand order; LDS rows are padded to 544 bytes, the stride at which that read is conflict-free.
+// Batches of at most 8 stage 8 rows (B columns 8..15 re-read rows 0..7 and feed outputs that are never stored).
 // ---------------------------------------------------------------------------------------------------------------
-// Batches of at most 8 leave MFMA B columns 8..15 unused, and with them the lanes that would load those columns.  Those
-// lanes fetch the operand of the FOLLOWING MFMA step instead: lane (col, q) reads batch row col % 8 at step offset col / 8,
-// so one instruction brings two steps and touches whole 128-byte lines; a DPP rotation of each 16-lane row by 8 then moves
-// the second step's data down to columns 0..7.  Columns 8..15 end up holding the other step's (real, finite) data and only
-// feed output columns that are never stored.  (Four or eight steps per load for batches <= 4 or <= 2 measured no faster.)
-template <int NT> __device__ __forceinline__ void load_x_paired(v8h (&x)[8][NT], const half_t *src)
-{
-#pragma unroll
-    for (int sl = 0; sl < 4; sl++) {
-        v4u v = *reinterpret_cast<const v4u *>(src + 64 * sl), w;
-#pragma unroll
-        for (int i = 0; i < 4; i++) w[i] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v[i], 0x128, 0xf, 0xf, false); // row_ror:8
-        x[2 * sl][0]     = __builtin_bit_cast(v8h, v);
-        x[2 * sl + 1][0] = __builtin_bit_cast(v8h, w);
-    }
-}
+constexpr int kXsRowBytes = 544;
 
-template <int FM, int NT, int RT> struct Stage {
+template <int FM, int RT> struct StageW {
     WFrag<FM> w[RT];
     uint32_t  g[RT]; // group exponents of the block (unused without them)
-    v8h       x[8][NT];
 };
 
-// How the activations of a K block are fetched: kXPaired (batches up to 8, block wholly inside K: two MFMA steps per load),
-// kXFull (block wholly inside K) or kXTail (the last block of a K that is not a multiple of 256).  The kernel chooses
-// outside its K loop: a choice made per block inside the loop cost 0.2 us of a 4.9 us launch at 4096 x 4096.
-enum XMode { kXPaired, kXFull, kXTail };
-
-template <int FM, bool GS, int NT, int RT, XMode MODE>
-__device__ __forceinline__ void load_stage(Stage<FM, NT, RT> &st, const uint8_t *wgroup, size_t tile_stride, const uint8_t *ggroup, uint32_t units,
-                                           uint32_t u, int lane, const half_t *const (&xrow)[NT], int q, uint32_t K, const half_t *xrow_packed)
+// LDS bytes per wavefront: the activation rows of one K block, or the RT*NT partial tiles of the epilogue (they share it)
+__host__ __device__ constexpr uint32_t stream_wave_bytes(int rows, int RT, int NT)
 {
-#pragma unroll
-    for (int r = 0; r < RT; r++) {
-        st.w[r] = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
-        st.g[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
-    }
-    // Every lane loads, without branches.  Batch columns beyond N read the last real row: an MFMA output column depends only
-    // on its own B column, and those columns are never stored.  K positions beyond K (only in the last block when K is not
-    // a multiple of 256) count as zero activations against the zero weights the native layout holds there (0 x 0, whatever
-    // the row holds elsewhere: an infinite activation must not meet a padding weight).
-    if constexpr (MODE == kXPaired) {
-        static_assert(NT == 1, "paired activation loads serve one column tile");
-        load_x_paired(st.x, xrow_packed + u * 256);
-    } else if constexpr (MODE == kXFull) { // one base address and immediate offsets
-#pragma unroll
-        for (int s = 0; s < 8; s++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) st.x[s][t] = *reinterpret_cast<const v8h *>(xrow[t] + u * 256 + 32 * s);
-    } else {
-#pragma unroll
-        for (int s = 0; s < 8; s++) {
-            uint32_t   k = u * 256 + 32 * s;
-            const bool beyond = k + 8 * q >= K; // such a piece is read at position 0 (a valid address) and replaced by zeros
-            if (beyond) k = 0;
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                v4u v = *reinterpret_cast<const v4u *>(xrow[t] + k);
-                st.x[s][t] = __builtin_bit_cast(v8h, beyond ? (v4u){ 0u, 0u, 0u, 0u } : v);
-            }
-        }
-    }
-    __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before the first conversion waits
-}
-
-template <int FM, bool GS, int NT, int RT>
-__device__ __forceinline__ void consume_stage(const Stage<FM, NT, RT> &st, v4f (&acc)[RT][NT])
-{
-#pragma unroll
-    for (int r = 0; r < RT; r++) {
-        AOps<FM> a;
-        convert<FM, GS>(st.w[r], a, st.g[r]);
-#pragma unroll
-        for (int s = 0; s < 8; s++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.s[s], st.x[s][t], acc[r][t], 0, 0, 0);
-    }
+    return (uint32_t)(rows * kXsRowBytes > RT * NT * 1024 ? rows * kXsRowBytes : RT * NT * 1024);
 }
 
 template <int FM, bool GS, int NT, int RT, int WAVES, bool SPLIT>
@@ -253,7 +195,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
                                                             uint32_t units, uint32_t splitK)
 {
-    __shared__ float red[WAVES][RT * NT][256];
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     // every kernel argument is fetched by one batch of scalar loads at the top (left alone, the compiler fetches them in
     // three batches, each a round trip to memory, as the code reaches their first use)
@@ -281,16 +223,6 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 #pragma unroll
         for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
 
-    const half_t *xrow[NT];
-#pragma unroll
-    for (int t = 0; t < NT; t++) {
-        uint32_t n = nbase + 16 * t + col;
-        xrow[t]    = X + (size_t)(n < N ? n : N - 1) * K + 8 * q;
-    }
-    // batches up to 8: two MFMA steps per activation load (see load_x_paired)
-    const int     prow = col & 7, pstep = col >> 3;
-    const half_t *xrow_packed = X + (size_t)((uint32_t)prow < N ? prow : N - 1) * K + 8 * q + 32 * pstep;
-
     // The epilogue gives thread e the output (row tile e/(256*NT), column tile, batch column, row e%16); its row scale is
     // fetched now so that no global load sits on the tail of the kernel.
     constexpr int kOutPerThread = (RT * NT * 256 + WAVES * kWave - 1) / (WAVES * kWave);
@@ -301,31 +233,132 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         my_scale[j] = scales[(R0 + (e < RT * NT * 256 ? (e >> 8) / NT : 0)) * 16 + (e & 15)];
     }
 
-    // workgroups that share an L2 (ids congruent mod 8) start on different K blocks, so that the chip does not ask
-    // the same activation lines of the same L2 channel at the same moment
+    const uint32_t ncols = N - nbase;              // batch columns of this column block that exist (the launcher made sure of >= 1)
+    const bool     small = NT == 1 && ncols <= 8;  // 8 rows are staged instead of 16
+    const uint32_t wave_bytes = small ? stream_wave_bytes(8, RT, NT) : stream_wave_bytes(16 * NT, RT, NT);
+    uint8_t       *mine = lds + wave * wave_bytes;  // this wavefront's LDS area
+
     // One K block at a time and no register double-buffering: the other wavefronts of the workgroup keep the memory system
     // busy while this one converts, and a second stage in registers measured slower at every size.
+    // workgroups that share an L2 (ids congruent mod 8) start on different K blocks, so that the chip does not ask
+    // the same activation lines of the same L2 channel at the same moment
     const uint32_t ufull = K / 256 < u1 ? K / 256 : u1; // the blocks before this one lie wholly inside K
     uint32_t       u = u0 + ((wave + (blockIdx.x >> 3)) % WAVES);
-    auto           run = [&](auto mode, uint32_t end) {
+    // MODE 0: batches up to 4 load in operand order (a quarter-wavefront then touches at most 4 lines, and the detour through
+    // LDS would only add latency); MODE 1: 8 rows through LDS; MODE 2: 16*NT rows through LDS.  TAIL: the block is cut by K
+    // (only the last block of a K that is no multiple of 256).  The kernel chooses outside its K loop: a choice made per
+    // block inside the loop cost 0.2 us of a 4.9 us launch.
+    auto run = [&](auto mode_c, auto tail_c, uint32_t end) {
+        constexpr int  MODE = decltype(mode_c)::value, ROWS = MODE == 2 ? 16 * NT : 8, LOADS = MODE == 0 ? 4 : ROWS / 2;
+        constexpr bool TAIL = decltype(tail_c)::value;
+        static_assert(!(MODE == 0 && (TAIL || NT != 1)), "operand-order loads serve whole blocks of one column tile");
+        // MODE 0: lane (col, q) reads batch row col % 8 at MFMA step offset col / 8
+        const uint32_t prow = (uint32_t)(col & 7) < ncols ? col & 7 : ncols - 1;
+        const half_t  *xpaired = X + (size_t)(nbase + prow) * K + 8 * q + 32 * (col >> 3);
+        // MODE 1, 2: load i of a block brings rows 2i and 2i+1, lane l takes bytes 16*(l%32).. of row 2i + l/32: a scalar base per
+        // load plus one per-lane offset for the whole kernel.  Rows beyond the batch repeat its last row (an MFMA output column
+        // depends only on its own B column, and those columns are never stored).
+        const uint8_t *xbase = reinterpret_cast<const uint8_t *>(X + (size_t)nbase * K);
+        const uint32_t off_one = (lane & 31) * 16, off_pair = (lane >> 5) * (K * 2) + off_one; // K < 2^31
+        uint8_t       *xw = mine + (lane >> 5) * kXsRowBytes + (lane & 31) * 16;
+        const uint8_t *xr = mine + (ROWS == 8 ? col & 7 : col) * kXsRowBytes + q * 16;
+        constexpr int  kWParts = Fmt<FM>::bits == 4 ? 2 : 3;
+        // Through LDS, the activation loads are issued BEFORE the weight loads: the memory pipeline returns loads in order, so
+        // activations asked for first are back (from L2) long before the weights (from HBM), and their trip through LDS
+        // is over when the weights arrive.  Issued after the weights they cost 5-10 % at batch 16.  In operand order they go
+        // between the second and the third weight load of the first row tile.
+        constexpr int kWBeforeX = MODE == 0 ? 2 : 0;
         for (; u < end; u += WAVES) {
-            Stage<FM, NT, RT> cur;
-            load_stage<FM, GS, NT, RT, decltype(mode)::value>(cur, wgroup, tile_stride, ggroup, units, u, lane, xrow, q, K, xrow_packed);
-            consume_stage<FM, GS, NT, RT>(cur, acc);
+            StageW<FM, RT> cur;
+            v4u            xv[LOADS];
+            auto           wpart = [&](int i) {
+                const int r = i / kWParts, part = i % kWParts;
+                load_wfrag_part<FM>(cur.w[r], wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
+            };
+#pragma unroll
+            for (int i = 0; i < kWBeforeX; i++) wpart(i);
+            // K positions beyond K count as zero activations against the zero weights the native layout holds there (0 x 0,
+            // whatever the row holds elsewhere: an infinite activation must not meet a padding weight): such a piece is read
+            // at the row's start (a valid address) and replaced by zeros
+            const bool beyond = TAIL && u * 256 + 8 * (lane & 31) >= K;
+#pragma unroll
+            for (int i = 0; i < LOADS; i++) {
+                if constexpr (MODE == 0) {
+                    xv[i] = *reinterpret_cast<const v4u *>(xpaired + (size_t)u * 256 + 64 * i);
+                } else {
+                    const uint32_t r0 = (uint32_t)(2 * i) < ncols ? 2 * i : ncols - 1;
+                    const uint8_t *sb = xbase + ((size_t)r0 * K + (size_t)u * 256) * 2;
+                    uint32_t       vo = (uint32_t)(2 * i + 1) < ncols ? off_pair : off_one;
+                    if (beyond) vo -= off_one;
+                    const v4u v = *reinterpret_cast<const v4u *>(sb + vo);
+                    xv[i] = beyond ? (v4u){ 0u, 0u, 0u, 0u } : v;
+                }
+            }
+#pragma unroll
+            for (int i = kWBeforeX; i < RT * kWParts; i++) wpart(i);
+#pragma unroll
+            for (int r = 0; r < RT; r++) cur.g[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
+            __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before anything waits
+            v8h x[8][NT];
+            if constexpr (MODE == 0) {
+                // one load brought two MFMA steps: a DPP rotation of each 16-lane row by 8 moves the second step's data down to
+                // columns 0..7 (columns 8..15 then hold the other step's real, finite data and feed outputs never stored)
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) {
+                    v4u w;
+#pragma unroll
+                    for (int i = 0; i < 4; i++) w[i] = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)xv[sl][i], 0x128, 0xf, 0xf, false); // row_ror:8
+                    x[2 * sl][0]     = __builtin_bit_cast(v8h, xv[sl]);
+                    x[2 * sl + 1][0] = __builtin_bit_cast(v8h, w);
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < LOADS; i++) *reinterpret_cast<v4u *>(xw + 2 * i * kXsRowBytes) = xv[i];
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+#pragma unroll
+                    for (int t = 0; t < NT; t++) x[s][t] = *reinterpret_cast<const v8h *>(xr + t * 16 * kXsRowBytes + 64 * s);
+                // the trip through LDS is issued before anything that waits for weights (left alone, the compiler moves register
+                // copies that feed the conversion above the LDS writes, and with them the wait for the weight loads)
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int r = 0; r < RT; r++) {
+                AOps<FM> a;
+                convert<FM, GS>(cur.w[r], a, cur.g[r]);
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+#pragma unroll
+                    for (int t = 0; t < NT; t++) acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a.s[s], x[s][t], acc[r][t], 0, 0, 0);
+            }
         }
     };
-    if (NT == 1 && N <= 8) {
-        if constexpr (NT == 1) run(std::integral_constant<XMode, kXPaired>{}, ufull);
+    typedef std::integral_constant<int, 0> Direct;
+    typedef std::integral_constant<int, 1> Staged8;
+    typedef std::integral_constant<int, 2> StagedAll;
+    auto staged = [&](auto mode_c, bool whole_blocks) {
+        if (whole_blocks) run(mode_c, std::false_type{}, ufull);
+        run(mode_c, std::true_type{}, u1); // at most one block, and only when K is not a multiple of 256
+    };
+    if (small) {
+        if constexpr (NT == 1) {
+            if (ncols <= 4) {
+                run(Direct{}, std::false_type{}, ufull);
+                staged(Staged8{}, false);
+            } else {
+                staged(Staged8{}, true);
+            }
+        }
     } else {
-        run(std::integral_constant<XMode, kXFull>{}, ufull);
+        staged(StagedAll{}, true);
     }
-    run(std::integral_constant<XMode, kXTail>{}, u1); // at most one block, and only when K is not a multiple of 256
 
-    // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col
+    // acc[r][t][i] = sum for output row 16r + 4q+i, batch column 16t+col.  Each wavefront parks its tiles in its own LDS
+    // area (its activation rows are dead by now; nobody else ever touched them), then the workgroup sums them.
 #pragma unroll
     for (int r = 0; r < RT; r++)
 #pragma unroll
-        for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[wave][r * NT + t][lane * 4]) = acc[r][t];
+        for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(mine + (r * NT + t) * 1024 + lane * 16) = acc[r][t];
     __syncthreads();
 
 #pragma unroll
@@ -337,7 +370,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
         int   idx = (((mm >> 2) * 16 + n) << 2) | (mm & 3);
         float sum = 0.f;
 #pragma unroll
-        for (int w = 0; w < WAVES; w++) sum += red[w][rt][idx];
+        for (int w = 0; w < WAVES; w++) sum += *reinterpret_cast<const float *>(lds + w * wave_bytes + rt * 1024 + idx * 4);
         uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
         if (ng < N) {
             float v = sum * ((float)my_scale[j] * Fmt<FM>::post_scale);
@@ -369,7 +402,222 @@ template <int FM, bool GS> __device__ __forceinline__ void convert_half(const WF
 // the conflict-free rate of 7 cycles per wavefront, against 8.8 cycles at 528 bytes and 32 cycles without padding.
 // The WK partial accumulators are summed through LDS at the end (WK > 1), then scaled and stored.
 // ---------------------------------------------------------------------------------------------------------------
-constexpr int kXsRowBytes = 544;
+
+// One segment of a tile's K range: K blocks [u0, u1) of row block `mb` against the batch columns from `nbase`, accumulated
+// into acc.  On return the wavefronts with wk == 0 hold the sums of all WK K-wavefronts; the LDS buffers are free again
+// once every wavefront of the workgroup has passed a barrier.
+template <int FM, bool GS, int NT, int RT, int WR, int WK>
+__device__ __forceinline__ void tile_segment(v4f (&acc)[RT][NT], const uint8_t *__restrict__ W, const uint8_t *__restrict__ gexp,
+                                             const half_t *__restrict__ X, uint32_t N, uint32_t K, uint32_t units, uint32_t mb, uint32_t nbase,
+                                             uint32_t u0, uint32_t u1, uint8_t *lds, int tid, int lane, int wr, int wk, int col, int q)
+{
+    constexpr int  TN = NT * 16, NTHREADS = WR * WK * kWave;
+    constexpr int  kBufBytes = WK * TN * kXsRowBytes;
+    constexpr int  kPieces = WK * TN * 32, kPerThread = (kPieces + NTHREADS - 1) / NTHREADS;
+    const uint32_t R0 = (mb * WR + wr) * RT; // first row tile of this wavefront
+    const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
+    const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
+    const uint8_t *ggroup = GS ? gexp + (size_t)R0 * units * 32 : nullptr;
+
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+
+    WFrag<FM> wcur[RT], wnxt[RT];
+    uint32_t  gcur[RT], gnxt[RT]; // group exponents travel with the weights (unused without them)
+    v4u       xr[kPerThread];
+
+    auto load_w = [&](WFrag<FM>(&dst)[RT], uint32_t(&gdst)[RT], uint32_t c0) {
+        const uint32_t u = c0 + wk;
+        if (u < u1) {
+#pragma unroll
+            for (int r = 0; r < RT; r++) {
+                dst[r]  = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
+                gdst[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
+            }
+        }
+    };
+    // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
+    // batch column (p/32) % TN, halfs 8*(p%32)..+7).  Row pointers and LDS offsets are fixed for the whole kernel.
+    // Columns beyond N read the last real row (their outputs are never stored); positions beyond K or beyond the split are
+    // read at position 0 of the row (a valid address) and staged as zeros (zero weights meet them, or no wavefront does).
+    const half_t *xrow[kPerThread];
+    uint32_t      xlds[kPerThread];
+#pragma unroll
+    for (int j = 0; j < kPerThread; j++) {
+        const uint32_t p = tid + NTHREADS * j, n = nbase + (p >> 5) % TN;
+        xrow[j] = X + (size_t)(n < N ? n : N - 1) * K + (p & 31) * 8 + (size_t)(p / (TN * 32)) * 256;
+        xlds[j] = (p >> 5) * kXsRowBytes + (p & 31) * 16;
+    }
+    // `full` (a compile-time flag): the whole chunk lies inside K and inside the segment, so every piece is a plain load.  The
+    // K loop below is written out per case: one choice per chunk inside the loop costs a wait for the activation loads before
+    // the weight loads can be issued.
+    auto load_x = [&](auto full, uint32_t c0) {
+        if constexpr (decltype(full)::value) {
+#pragma unroll
+            for (int j = 0; j < kPerThread; j++)
+                if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
+        } else {
+#pragma unroll
+            for (int j = 0; j < kPerThread; j++) {
+                const uint32_t p = tid + NTHREADS * j;
+                if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
+                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
+                    const bool     ok = k < K && u < u1;
+                    const v4u      v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                    xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
+                }
+            }
+        }
+    };
+    // The same loads one at a time (i = 0 .. kLoads-1: weights first, then activation pieces).  The 256 x 128 tile spreads them
+    // over its MFMA steps instead of issuing them in one burst: measured 10-12 % faster for batches from 1024 up (the burst keeps
+    // a wavefront, which issues in order, from starting its MFMAs until the CU has accepted its last load); for the smaller
+    // tiles, with fewer MFMAs between two loads, spreading measured 0-8 % slower and they keep the burst.
+    constexpr bool kSpreadLoads = NT >= 8 && WR * WK >= 8;
+    constexpr int  kWParts = Fmt<FM>::bits == 4 ? 2 : 3, kWLoads = RT * kWParts, kLoads = kWLoads + kPerThread, kPerStep = (kLoads + 7) / 8;
+    auto load_one = [&](auto full, int i, uint32_t c0) {
+        if (i < kWLoads) {
+            const int      r = i / kWParts, part = i % kWParts;
+            const uint32_t u = c0 + wk;
+            if (u < u1) {
+                load_wfrag_part<FM>(wnxt[r], wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
+                if (part == 0) gnxt[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
+            }
+        } else if (i < kLoads) {
+            const int      j = i - kWLoads;
+            const uint32_t p = tid + NTHREADS * j;
+            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
+                if constexpr (decltype(full)::value) {
+                    xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
+                } else {
+                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
+                    const bool     ok = k < K && u < u1;
+                    const v4u      v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
+                    xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
+                }
+            }
+        }
+    };
+    auto store_x = [&](int buf) {
+#pragma unroll
+        for (int j = 0; j < kPerThread; j++)
+            if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) *reinterpret_cast<v4u *>(lds + buf * kBufBytes + xlds[j]) = xr[j];
+    };
+    typedef std::integral_constant<int, 0> NoNext;       // the last chunk: nothing to fetch
+    typedef std::integral_constant<int, 1> FullNext;     // the next chunk is a full one
+    typedef std::integral_constant<int, 2> PartialNext;  // the next chunk is cut by K or by the end of the segment
+    typedef std::integral_constant<bool, true> Full;
+    typedef std::integral_constant<bool, false> Partial;
+
+    if (u0 < u1) {
+        const uint32_t ufull = K / 256 < u1 ? K / 256 : u1; // chunks that end at or before this block are full
+        if (u0 + WK <= ufull)
+            load_x(Full{}, u0);
+        else
+            load_x(Partial{}, u0);
+        load_w(wcur, gcur, u0);
+        store_x(0);
+        __syncthreads();
+        int      buf = 0;
+        uint32_t c0 = u0;
+        // one chunk: fetch the next one (if any), compute this one, stage the next one's activations, barrier
+        auto chunk = [&](auto next) {
+            constexpr int  kNext = decltype(next)::value;
+            constexpr bool more = kNext != 0;
+            typedef std::integral_constant<bool, kNext == 1> NextIsFull;
+            if (more && (!kSpreadLoads || c0 + wk >= u1)) { // (a wavefront without a K block in this chunk has no MFMAs to spread over)
+                load_x(NextIsFull{}, c0 + WK);
+                load_w(wnxt, gnxt, c0 + WK);
+            }
+            if (c0 + wk < u1) {
+                const uint8_t *xs = lds + buf * kBufBytes + (wk * TN + col) * kXsRowBytes + q * 16;
+                v8h            a0[RT][4], a1[RT][4];
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 0, a0[r], gcur[r]);
+                // second half converted ahead of the first half's MFMAs: the VALU work then runs under the matrix pipe
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 1, a1[r], gcur[r]);
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        v8h b[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xs + t * 16 * kXsRowBytes + (4 * h + s) * 64);
+#pragma unroll
+                        for (int r = 0; r < RT; r++)
+#pragma unroll
+                            for (int t = 0; t < NT; t++)
+                                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h == 0 ? a0[r][s] : a1[r][s], b[t], acc[r][t], 0, 0, 0);
+                        if constexpr (kSpreadLoads && more) {
+#pragma unroll
+                            for (int i = (4 * h + s) * kPerStep; i < (4 * h + s + 1) * kPerStep; i++) load_one(NextIsFull{}, i, c0 + WK);
+                        }
+                    }
+                }
+            }
+            if (more) {
+                store_x(buf ^ 1); // that buffer was last read before the barrier that ended the previous iteration
+#pragma unroll
+                for (int r = 0; r < RT; r++) wcur[r] = wnxt[r], gcur[r] = gnxt[r];
+            }
+            __syncthreads();
+            c0 += WK, buf ^= 1;
+        };
+        while (c0 + 2 * WK <= ufull) chunk(FullNext{});
+        while (c0 + WK < u1) chunk(PartialNext{});
+        chunk(NoNext{});
+    }
+
+    // acc[r][t][i]: output row (R0+r)*16 + 4q+i, batch column nbase + 16t + col
+    if (WK > 1) {
+        float *red = reinterpret_cast<float *>(lds); // [WK][WR][RT*NT][256]; the last barrier above freed the buffers
+#pragma unroll
+        for (int r = 0; r < RT; r++)
+#pragma unroll
+            for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[(((wk * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]) = acc[r][t];
+        __syncthreads();
+        if (wk == 0) {
+#pragma unroll
+            for (int r = 0; r < RT; r++)
+#pragma unroll
+                for (int t = 0; t < NT; t++)
+#pragma unroll
+                    for (int k2 = 1; k2 < WK; k2++)
+                        acc[r][t] += *reinterpret_cast<const v4f *>(&red[(((k2 * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]);
+        }
+    }
+}
+
+// Scales the sums of one wavefront's RT x NT output tiles and stores them: fp16 into C, or fp32 partial sums into `part`
+// ([N][M] floats) when that is not null.  acc[r][t][i]: output row (R0+r)*16 + 4q+i, batch column nbase + 16t + col.
+typedef _Float16 v4h __attribute__((ext_vector_type(4)));
+template <int FM, int NT, int RT>
+__device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], half_t *__restrict__ C, float *__restrict__ part, uint32_t M,
+                                           uint32_t N, uint32_t R0, uint32_t nbase, int col, int q)
+{
+#pragma unroll
+    for (int r = 0; r < RT; r++) {
+        const uint32_t mg = (R0 + r) * 16 + 4 * q;
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            const uint32_t ng = nbase + 16 * t + col;
+            if (ng < N) {
+                v4f v;
+#pragma unroll
+                for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
+                if (!part) {
+                    v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
+                    *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
+                } else {
+                    *reinterpret_cast<v4f *>(part + (size_t)ng * M + mg) = v;
+                }
+            }
+        }
+    }
+}
 
 template <int FM, bool GS, int NT, int RT, int WR, int WK>
 __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
@@ -401,195 +649,16 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         u1 = u0 + avg + (split < extra ? 1u : 0u);
     }
 
-    const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
-    const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
-    const uint8_t *ggroup = GS ? gexp + (size_t)R0 * units * 32 : nullptr;
-
     v4f acc[RT][NT];
-#pragma unroll
-    for (int r = 0; r < RT; r++)
-#pragma unroll
-        for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
-
-    WFrag<FM> wcur[RT], wnxt[RT];
-    uint32_t  gcur[RT], gnxt[RT]; // group exponents travel with the weights (unused without them)
-    v4u       xr[kPerThread];
-
     // row scales of this lane's outputs (rows 4q..4q+3 of each of its row tiles), fetched before the main loop so that no
     // global load sits on the tail of the kernel
-    typedef _Float16 v4h __attribute__((ext_vector_type(4)));
     v4h sc4[RT];
 #pragma unroll
     for (int r = 0; r < RT; r++) sc4[r] = *reinterpret_cast<const v4h *>(scales + (R0 + r) * 16 + 4 * q);
 
-    auto load_w = [&](WFrag<FM>(&dst)[RT], uint32_t(&gdst)[RT], uint32_t c0) {
-        const uint32_t u = c0 + wk;
-        if (u < u1) {
-#pragma unroll
-            for (int r = 0; r < RT; r++) {
-                dst[r]  = load_wfrag<FM>(wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane);
-                gdst[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
-            }
-        }
-    };
-    // Per-thread pieces of the activation chunk: piece p = tid + NTHREADS*j is 16 bytes, (K block p / (TN*32) of the chunk,
-    // batch column (p/32) % TN, halfs 8*(p%32)..+7).  Row pointers and LDS offsets are fixed for the whole kernel.
-    // Columns beyond N read the last real row (their outputs are never stored); positions beyond K or beyond the split are
-    // read at position 0 of the row (a valid address) and staged as zeros (zero weights meet them, or no wavefront does).
-    const half_t *xrow[kPerThread];
-    uint32_t      xlds[kPerThread];
-#pragma unroll
-    for (int j = 0; j < kPerThread; j++) {
-        const uint32_t p = tid + NTHREADS * j, n = nbase + (p >> 5) % TN;
-        xrow[j] = X + (size_t)(n < N ? n : N - 1) * K + (p & 31) * 8 + (size_t)(p / (TN * 32)) * 256;
-        xlds[j] = (p >> 5) * kXsRowBytes + (p & 31) * 16;
-    }
-    auto load_x = [&](uint32_t c0) {
-        if ((c0 + WK) * 256 <= K && c0 + WK <= u1) { // uniform: the whole chunk lies inside K and inside the split
-#pragma unroll
-            for (int j = 0; j < kPerThread; j++)
-                if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
-        } else {
-#pragma unroll
-            for (int j = 0; j < kPerThread; j++) {
-                const uint32_t p = tid + NTHREADS * j;
-                if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
-                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
-                    const bool     ok = k < K && u < u1;
-                    {
-                        const v4u v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
-                        xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
-                    }
-                }
-            }
-        }
-    };
-    // The same loads one at a time (i = 0 .. kLoads-1: weights first, then activation pieces).  The 256 x 128 tile spreads them
-    // over its MFMA steps instead of issuing them in one burst: measured 10-12 % faster for batches from 1024 up (the burst keeps
-    // a wavefront, which issues in order, from starting its MFMAs until the CU has accepted its last load); for the smaller
-    // tiles, with fewer MFMAs between two loads, spreading measured 0-8 % slower and they keep the burst.
-    constexpr bool kSpreadLoads = NT >= 8 && WR * WK >= 8;
-    constexpr int  kWParts = Fmt<FM>::bits == 4 ? 2 : 3, kWLoads = RT * kWParts, kLoads = kWLoads + kPerThread, kPerStep = (kLoads + 7) / 8;
-    auto load_one = [&](int i, uint32_t c0) {
-        if (i < kWLoads) {
-            const int      r = i / kWParts, part = i % kWParts;
-            const uint32_t u = c0 + wk;
-            if (u < u1) {
-                load_wfrag_part<FM>(wnxt[r], wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
-                if (part == 0) gnxt[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
-            }
-        } else if (i < kLoads) {
-            const int      j = i - kWLoads;
-            const uint32_t p = tid + NTHREADS * j;
-            if (kPieces % NTHREADS == 0 || p < (uint32_t)kPieces) {
-                if ((c0 + WK) * 256 <= K && c0 + WK <= u1) { // uniform
-                    xr[j] = *reinterpret_cast<const v4u *>(xrow[j] + (size_t)c0 * 256);
-                } else {
-                    const uint32_t u = c0 + p / (TN * 32), k = u * 256 + (p & 31) * 8;
-                    const bool     ok = k < K && u < u1;
-                    {
-                        const v4u v = *reinterpret_cast<const v4u *>(ok ? xrow[j] + (size_t)c0 * 256 : xrow[j] - ((p & 31) * 8 + (size_t)(p / (TN * 32)) * 256));
-                        xr[j] = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
-                    }
-                }
-            }
-        }
-    };
-    auto store_x = [&](int buf) {
-#pragma unroll
-        for (int j = 0; j < kPerThread; j++)
-            if (kPieces % NTHREADS == 0 || tid + NTHREADS * j < kPieces) *reinterpret_cast<v4u *>(lds + buf * kBufBytes + xlds[j]) = xr[j];
-    };
+    tile_segment<FM, GS, NT, RT, WR, WK>(acc, W, gexp, X, N, K, units, mb, nbase, u0, u1, lds, tid, lane, wr, wk, col, q);
 
-    if (u0 < u1) {
-        load_x(u0);
-        load_w(wcur, gcur, u0);
-        store_x(0);
-        __syncthreads();
-        int buf = 0;
-        for (uint32_t c0 = u0; c0 < u1; c0 += WK, buf ^= 1) {
-            const bool more = c0 + WK < u1;
-            if (more && (!kSpreadLoads || c0 + wk >= u1)) { // (a wavefront without a K block in this chunk has no MFMAs to spread over)
-                load_x(c0 + WK);
-                load_w(wnxt, gnxt, c0 + WK);
-            }
-            if (c0 + wk < u1) {
-                const uint8_t *xs = lds + buf * kBufBytes + (wk * TN + col) * kXsRowBytes + q * 16;
-                v8h            a0[RT][4], a1[RT][4];
-#pragma unroll
-                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 0, a0[r], gcur[r]);
-                // second half converted ahead of the first half's MFMAs: the VALU work then runs under the matrix pipe
-#pragma unroll
-                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wcur[r], 1, a1[r], gcur[r]);
-#pragma unroll
-                for (int h = 0; h < 2; h++) {
-#pragma unroll
-                    for (int s = 0; s < 4; s++) {
-                        v8h b[NT];
-#pragma unroll
-                        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xs + t * 16 * kXsRowBytes + (4 * h + s) * 64);
-#pragma unroll
-                        for (int r = 0; r < RT; r++)
-#pragma unroll
-                            for (int t = 0; t < NT; t++)
-                                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h == 0 ? a0[r][s] : a1[r][s], b[t], acc[r][t], 0, 0, 0);
-                        if constexpr (kSpreadLoads) {
-                            if (more) {
-#pragma unroll
-                                for (int i = (4 * h + s) * kPerStep; i < (4 * h + s + 1) * kPerStep; i++) load_one(i, c0 + WK);
-                            }
-                        }
-                    }
-                }
-            }
-            if (more) {
-                store_x(buf ^ 1); // that buffer was last read before the barrier that ended the previous iteration
-#pragma unroll
-                for (int r = 0; r < RT; r++) wcur[r] = wnxt[r], gcur[r] = gnxt[r];
-            }
-            __syncthreads();
-        }
-    }
-
-    // acc[r][t][i]: output row (R0+r)*16 + 4q+i, batch column nbase + 16t + col
-    if (WK > 1) {
-        float *red = reinterpret_cast<float *>(lds); // [WK][WR][RT*NT][256]; the last barrier above freed the buffers
-#pragma unroll
-        for (int r = 0; r < RT; r++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) *reinterpret_cast<v4f *>(&red[(((wk * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]) = acc[r][t];
-        __syncthreads();
-        if (wk == 0) {
-#pragma unroll
-            for (int r = 0; r < RT; r++)
-#pragma unroll
-                for (int t = 0; t < NT; t++)
-#pragma unroll
-                    for (int k2 = 1; k2 < WK; k2++)
-                        acc[r][t] += *reinterpret_cast<const v4f *>(&red[(((k2 * WR + wr) * RT + r) * NT + t) * 256 + lane * 4]);
-        }
-    }
-    if (wk == 0) {
-#pragma unroll
-        for (int r = 0; r < RT; r++) {
-            const uint32_t mg = (R0 + r) * 16 + 4 * q;
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                const uint32_t ng = nbase + 16 * t + col;
-                if (ng < N) {
-                    v4f v;
-#pragma unroll
-                    for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
-                    if (splitK == 1) {
-                        v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
-                        *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
-                    } else {
-                        *reinterpret_cast<v4f *>(ws + ((size_t)split * N + ng) * M + mg) = v;
-                    }
-                }
-            }
-        }
-    }
+    if (wk == 0) tile_store<FM, NT, RT>(acc, sc4, C, splitK == 1 ? nullptr : ws + (size_t)split * N * M, M, N, R0, nbase, col, q);
 }
 
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
@@ -849,22 +918,41 @@ __global__ __launch_bounds__(256) void quant_to_native(uint8_t *__restrict__ nat
 }
 // ------------------------------------------------------------------------------------------------ launch helpers
 
+// Lets `Kernel` use up to `bytes` of dynamic LDS.  The attribute belongs to the device's copy of the kernel: set once per device.
+template <auto Kernel> int allow_dynamic_lds(size_t bytes)
+{
+    static std::atomic<uint64_t> attr_set{ 0 }; // bit d: done on device d; setting it twice is harmless, so no lock
+    int                          dev = 0;
+    if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
+    const uint64_t bit = dev >= 0 && dev < 64 ? 1ull << dev : 0;
+    if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+        if (e != hipSuccess) return (int)e;
+        attr_set.fetch_or(bit, std::memory_order_relaxed);
+    }
+    return 0;
+}
+
 template <int FM, bool GS, int NT, int RT, int WAVES>
 int launch_stream(hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
                   int splitK)
 {
-    uint32_t units = (uint32_t)((K + 255) / 256);
-    dim3     grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
-    auto     go = [&](auto kernel) {
-        hipLaunchKernelGGL(kernel, grid, dim3(WAVES * kWave), 0, st, static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc),
+    constexpr size_t kMaxLds = (size_t)WAVES * stream_wave_bytes(16 * NT, RT, NT);
+    static_assert(kMaxLds <= 160 * 1024, "the wavefronts' activation rows do not fit in LDS");
+    uint32_t     units = (uint32_t)((K + 255) / 256);
+    dim3         grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
+    const size_t lds_bytes = NT == 1 && N <= 8 ? (size_t)WAVES * stream_wave_bytes(8, RT, NT) : kMaxLds;
+    auto         go = [&](auto kernel_c) -> int {
+        constexpr auto kernel = decltype(kernel_c)::value;
+        if (kMaxLds > 48 * 1024)
+            if (int rc = allow_dynamic_lds<kernel>(kMaxLds)) return rc;
+        hipLaunchKernelGGL(kernel, grid, dim3(WAVES * kWave), lds_bytes, st, static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc),
                            static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B), static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N,
                            (uint32_t)K, units, (uint32_t)splitK);
+        return (int)hipGetLastError();
     };
-    if (splitK > 1)
-        go(gemm_stream<FM, GS, NT, RT, WAVES, true>);
-    else
-        go(gemm_stream<FM, GS, NT, RT, WAVES, false>);
-    return (int)hipGetLastError();
+    if (splitK > 1) return go(std::integral_constant<decltype(&gemm_stream<FM, GS, NT, RT, WAVES, true>), &gemm_stream<FM, GS, NT, RT, WAVES, true>>{});
+    return go(std::integral_constant<decltype(&gemm_stream<FM, GS, NT, RT, WAVES, false>), &gemm_stream<FM, GS, NT, RT, WAVES, false>>{});
 }
 
 template <int FM, bool GS, int NT, int RT, int WR, int WK>
@@ -876,18 +964,8 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *gexp,
     constexpr size_t lds_bytes = x_bytes > red_bytes ? x_bytes : red_bytes;
     static_assert(lds_bytes <= 160 * 1024, "tile does not fit in LDS");
     if (M % TM) return FP6MI_ERR_SHAPE;
-    if (lds_bytes > 48 * 1024) { // the attribute belongs to the device's copy of the kernel: once per device
-        static std::atomic<uint64_t> attr_set{ 0 }; // bit d: done on device d; setting it twice is harmless, so no lock
-        int                          dev = 0;
-        if (hipError_t e = hipGetDevice(&dev); e != hipSuccess) return (int)e;
-        const uint64_t bit = dev < 64 ? 1ull << dev : 0;
-        if (!(attr_set.load(std::memory_order_relaxed) & bit)) {
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_tile<FM, GS, NT, RT, WR, WK>),
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-            if (e != hipSuccess) return (int)e;
-            attr_set.fetch_or(bit, std::memory_order_relaxed);
-        }
-    }
+    if (lds_bytes > 48 * 1024)
+        if (int rc = allow_dynamic_lds<&gemm_tile<FM, GS, NT, RT, WR, WK>>(lds_bytes)) return rc;
     uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
     size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
     if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
@@ -909,8 +987,6 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
         FP6MI_CASE(2, 1, 4) FP6MI_CASE(2, 1, 8)
         FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
-        FP6MI_CASE(4, 1, 4) FP6MI_CASE(4, 1, 8)
-        FP6MI_CASE(4, 2, 4) FP6MI_CASE(4, 2, 8)
 #undef FP6MI_CASE
     } else if (c.kind == 1) {
 #define FP6MI_CASE(NT, RT, WR, WK) \

@@ -34,7 +34,7 @@ FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit
 # ever came within 3 % of the best in exhaustive sweeps
 COMPILED_STREAM = [(0, nt, rt, 1, wk) for (nt, rt, wk) in
                    [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 4, 4), (1, 4, 8), (2, 1, 4), (2, 1, 8), (2, 2, 4),
-                    (2, 2, 8), (4, 1, 4), (4, 1, 8), (4, 2, 4), (4, 2, 8)]]
+                    (2, 2, 8)]]
 COMPILED_TILE = [(1,) + c for c in
                  [(2, 1, 4, 4), (2, 2, 4, 4), (2, 2, 4, 2), (2, 2, 4, 1), (2, 4, 4, 1), (2, 4, 4, 2), (4, 2, 4, 2), (4, 2, 4, 1), (4, 4, 4, 1),
                   (4, 4, 2, 1), (4, 4, 2, 2), (8, 2, 4, 1), (8, 2, 2, 1), (4, 2, 8, 1), (4, 2, 8, 2), (2, 2, 8, 1), (2, 2, 8, 2), (8, 2, 8, 1),

@@ -276,7 +276,7 @@ def test_c_abi_drop_in_second_stream_and_capture():
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
-@pytest.mark.parametrize("N", [8, 16, 40])
+@pytest.mark.parametrize("N", [1, 3, 4, 5, 8, 9, 13, 16, 40])
 def test_infinite_activation_next_to_padded_columns(E, M, N):
     """K = 320 leaves 192 padding columns in the last 256-column block of the native layout.  An infinite activation in
     column 0 must give infinite outputs of the right sign (where the weight of column 0 is not zero), not NaN from
@@ -295,6 +295,22 @@ def test_infinite_activation_next_to_padded_columns(E, M, N):
     assert nz.sum() > OC // 2
     assert np.array_equal(np.isnan(y), np.isnan(ref)) and not np.isnan(y[:, nz]).any()
     assert np.array_equal(y[:, nz], ref[:, nz])       # +-inf, exactly
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("cfg,N", [((0, 1, 1, 1, 16), 3), ((0, 1, 2, 1, 8), 7), ((0, 1, 4, 1, 4), 11), ((0, 1, 2, 1, 16), 16), ((0, 2, 1, 1, 8), 19),
+                                   ((0, 2, 2, 1, 4), 32), ((0, 2, 2, 1, 8), 41), ((0, 1, 1, 1, 8), 21)])
+def test_stream_shapes_with_a_cut_last_block(E, M, cfg, N):
+    """The small-batch kernel's three ways of fetching activations (operand order up to batch 4, 8 rows or all rows of the
+    column block through LDS beyond), each on whole K blocks and on a last block cut by K (K = 1344 = 5.25 blocks), with
+    batches that leave the last row pair and the last column block partly empty, with and without a split."""
+    print("case stream tail", E, M, cfg, N, flush=True)
+    OC, IC = 512, 1344
+    raw, sc, x = synth.uniform_problem(7300 + N, OC, IC, N, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    for splitK in (1, 2):
+        check_close(gemm_capi(E, M, native, scd, xd, OC, splitK, cfg), ref, "cfg %s N %d splitK %d" % (cfg, N, splitK))
 
 
 def test_torch_extension_and_ctypes_binding_agree(monkeypatch):
