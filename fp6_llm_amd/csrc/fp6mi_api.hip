@@ -106,9 +106,12 @@ inline double tile_estimate_ns(size_t M, size_t N, size_t K, int splitK, int cus
 
 // ---- measured launch shapes (generated by `python -m fp6_llm_amd.tune`, MI355X, 256 CUs) ----
 struct TuneCfg { uint8_t kind, nt, rt, wr, wk; uint16_t t; };              // t in 0.02 us; kind 255 = not measured
-struct TuneEntry { uint8_t xb; uint16_t m256, k64, n; TuneCfg sk[4]; };    // sk[i]: best shape for splitK = 1 << i
+constexpr int kSplits[] = { 1, 2, 3, 4, 6, 8 };                             // the splits the table knows
+constexpr int kNumSplits = sizeof(kSplits) / sizeof(kSplits[0]);
+inline int split_index(int splitK) { for (int i = 0; i < kNumSplits; i++) if (kSplits[i] == splitK) return i; return -1; }
+struct TuneEntry { uint8_t xb; uint16_t m256, k64, n; TuneCfg sk[kNumSplits]; };    // sk[i]: best shape for splitK = kSplits[i]
 const TuneEntry kTune[] = {
-    { 0, 0, 0, 0, { { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 } } }, // keeps the array non-empty
+    { 0, 0, 0, 0, { { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 }, { 255, 0, 0, 0, 0, 0 } } }, // keeps the array non-empty
 #include "fp6mi_tuning.inc"
 };
 
@@ -122,7 +125,7 @@ inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (
 // 16384 and 17920 rows differ by 9 % in size but by a whole round of 64-row workgroups; sweeps off the grid showed that
 // this, not the distance, decides which neighbour's shape is right.  Farther neighbours pay 15 % per octave of distance.
 struct TuneGroup { int xb; size_t n, begin, end; }; // entries [begin, end) of kTune share format and batch (the table is sorted by them)
-struct TuneAnswer { bool valid; LaunchCfg cfg[4]; float t[4]; }; // index i: splitK = 1 << i; t in 0.02 us, 0 = no proposal
+struct TuneAnswer { bool valid; LaunchCfg cfg[kNumSplits]; float t[kNumSplits]; }; // index i: splitK = kSplits[i]; t in 0.02 us, 0 = no proposal
 
 const std::vector<TuneGroup> &tune_groups()
 {
@@ -185,11 +188,11 @@ const TuneAnswer *tune_lookup(int xbits, size_t M, size_t N, size_t K)
     for (int j = 0; j < count; j++) {
         const TuneEntry &e = *near[j];
         const size_t     Me = (size_t)e.m256 * 256, Ke = (size_t)e.k64 * 64, Nq = N > group->n ? N : group->n;
-        for (int i = 0; i < 4; i++) {
+        for (int i = 0; i < kNumSplits; i++) {
             const TuneCfg &c = e.sk[i];
-            if (!cfg_fits(c, M) || (size_t)(1 << i) > units) continue;
+            if (!cfg_fits(c, M) || (size_t)kSplits[i] > units) continue;
             double t = (double)c.t * (double)K / (double)Ke * (1.0 + 0.15 * dist[j]);
-            t *= rounds_on_chip(c, M, Nq, 1 << i) / rounds_on_chip(c, Me, group->n, 1 << i);
+            t *= rounds_on_chip(c, M, Nq, kSplits[i]) / rounds_on_chip(c, Me, group->n, kSplits[i]);
             if (a.t[i] == 0.f || (float)t < a.t[i]) {
                 a.t[i] = (float)t;
                 a.cfg[i] = LaunchCfg{ c.kind, c.nt, c.rt, c.wr, c.wk };
@@ -209,9 +212,8 @@ const TuneAnswer *tune_lookup(int xbits, size_t M, size_t N, size_t K)
 inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, int cus)
 {
     LaunchCfg c;
-    if (cus == 256 && (splitK == 1 || splitK == 2 || splitK == 4 || splitK == 8)) {
+    if (const int i = split_index(splitK); cus == 256 && i >= 0) {
         if (const TuneAnswer *a = tune_lookup(xbits, M, N, K)) {
-            const int i = splitK == 1 ? 0 : splitK == 2 ? 1 : splitK == 4 ? 2 : 3;
             if (a->t[i] > 0.f) return a->cfg[i];
         }
     }
@@ -339,9 +341,9 @@ static int heuristic_splitk(int xbits, size_t M, size_t N, size_t K, int num_cus
         if (const TuneAnswer *a = tune_lookup(xbits, M, N, K)) {
             int   best_s = 0;
             float best_t = 0.f;
-            for (int i = 0; i < 4; i++) {
+            for (int i = 0; i < kNumSplits; i++) {
                 if (a->t[i] == 0.f) continue;
-                if (best_s == 0 || a->t[i] * 1.03f < best_t) { best_s = 1 << i; best_t = a->t[i]; }
+                if (best_s == 0 || a->t[i] * 1.03f < best_t) { best_s = kSplits[i]; best_t = a->t[i]; }
             }
             if (best_s) return best_s;
         }

@@ -6,6 +6,8 @@ This tool measures every candidate shape on the GPU it runs on and writes that t
 
     python -m fp6_llm_amd.tune sweep --format 6 --out fp6_llm_amd/tuning/fp6_mi355x.jsonl      # minutes of GPU time
     python -m fp6_llm_amd.tune compact fp6_llm_amd/tuning/*.jsonl                               # after re-measuring with --append
+    python -m fp6_llm_amd.tune sweep --format 6 --kinds stream --n 8,12,16 --out part.jsonl     # after a change to one kernel:
+    python -m fp6_llm_amd.tune merge fp6_llm_amd/tuning/fp6_mi355x.jsonl part.jsonl             #   only its candidates are re-measured
     python -m fp6_llm_amd.tune emit fp6_llm_amd/tuning/*.jsonl                                  # -> csrc/fp6mi_tuning.inc
     python -m fp6_llm_amd.build
 
@@ -27,7 +29,7 @@ STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 4) for wk in (4, 8, 16) if (r
 STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4)]                      # two 16-column tiles per workgroup, batches 17..32
 TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
         (1, 8, 2, 8, 1)]
-SPLITS = (1, 2, 4, 8)
+SPLITS = (1, 2, 3, 4, 6, 8)      # 3 and 6 fill 256 CUs where 80 or 40 row blocks leave a power of two short (M = 10240, 5120)
 FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit width
 
 # every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip, the same for every format); the candidates above are the ones that
@@ -66,7 +68,17 @@ def tile_rows(cfg):
     return 16 * rt * (wr if kind == 1 else 1)
 
 
-def candidates(OC, IC, BS):
+def candidates(OC, IC, BS, kinds=None, splits=None):
+    """(shape, splitK) pairs worth measuring; `kinds` ("stream", "tile") and `splits` narrow the list for a partial sweep."""
+    for cfg, sk in _all_candidates(OC, IC, BS):
+        if kinds and ("stream" if cfg[0] == 0 else "tile") not in kinds:
+            continue
+        if splits and sk not in splits:
+            continue
+        yield cfg, sk
+
+
+def _all_candidates(OC, IC, BS):
     if BS <= 16:
         cfgs = STREAM_SMALL
     else:
@@ -155,6 +167,8 @@ def sweep(args):
         problems = [tuple(int(v) for v in p.split("x")) for p in args.pairs.split(",")]
     else:
         problems = [(OC, IC) for OC in Ms for IC in Ks]
+    kinds = set(args.kinds.split(",")) if args.kinds else None
+    splits = set(int(v) for v in args.splits.split(",")) if args.splits else None
     bench = Bench(args.iters, args.reps)
     os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
     with open(args.out, "a" if args.append else "w") as f:
@@ -164,11 +178,14 @@ def sweep(args):
                     continue
                 for BS in Ns:
                     best = {}
-                    for cfg, sk in candidates(OC, IC, BS):
+                    for cfg, sk in candidates(OC, IC, BS, kinds, splits):
                         t = bench(E, M, OC, IC, BS, cfg, sk)
                         if t is not None and (str(sk) not in best or t < best[str(sk)][1]):
                             best[str(sk)] = [list(cfg), round(t, 3)]
-                    f.write(json.dumps({"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best}) + "\n")
+                    row = {"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best}
+                    if kinds or splits:   # a partial row: `merge` folds it into a full one
+                        row["partial"] = {"kinds": sorted(kinds) if kinds else ["stream", "tile"], "splits": sorted(splits) if splits else list(SPLITS)}
+                    f.write(json.dumps(row) + "\n")
                     f.flush()
                     print("e%dm%d %dx%d N=%d: " % (E, M, OC, IC, BS) + "  ".join("sk%s %s %.2f" % (k, "".join(map(str, v[0])), v[1]) for k, v in best.items()),
                           flush=True)
@@ -181,11 +198,11 @@ def emit(args):
             r = json.loads(line)
             rows[(1 + r["E"] + r["M"], r["BS"], r["OC"], r["IC"])] = r   # later files override earlier ones
     lines = ["// Measured launch shapes: generated by `python -m fp6_llm_amd.tune emit`; do not edit by hand.",
-             "// {bits, M/256, K/64, N, {best shape for splitK 1, 2, 4, 8: kind, n_tiles, row_tiles, row_waves, k_waves, time in 0.02 us}}"]
+             "// {bits, M/256, K/64, N, {best shape for splitK 1, 2, 3, 4, 6, 8: kind, n_tiles, row_tiles, row_waves, k_waves, time in 0.02 us}}"]
     for (xb, BS, OC, IC) in sorted(rows):
         r = rows[(xb, BS, OC, IC)]
         cells = []
-        for sk in ("1", "2", "4", "8"):
+        for sk in (str(v) for v in SPLITS):
             if sk in r["best"]:
                 cfg, t = r["best"][sk]
                 cells.append("{%d,%d,%d,%d,%d,%d}" % (*cfg, min(65535, int(round(t / 0.02)))))
@@ -195,6 +212,37 @@ def emit(args):
     with open(INC_PATH, "w") as f:
         f.write("\n".join(lines) + "\n")
     print("%d entries -> %s" % (len(rows), INC_PATH))
+
+
+def merge(args):
+    """Folds partial rows (sweeps with --kinds / --splits) into the full measurement file: within the kinds and splits a
+    partial row covers, the old entry is stale and gives way; elsewhere the faster of the two stands."""
+    rows = {}
+    for line in open(args.main):
+        r = json.loads(line)
+        rows[(r["E"], r["M"], r["OC"], r["IC"], r["BS"])] = r
+    changed = 0
+    for path in args.parts:
+        for line in open(path):
+            p = json.loads(line)
+            key = (p["E"], p["M"], p["OC"], p["IC"], p["BS"])
+            part = p.get("partial", {"kinds": ["stream", "tile"], "splits": list(SPLITS)})
+            old = rows.get(key, {"E": p["E"], "M": p["M"], "OC": p["OC"], "IC": p["IC"], "BS": p["BS"], "best": {}})
+            best = {}
+            for sk in sorted(set(old["best"]) | set(p["best"]), key=int):
+                o, n = old["best"].get(sk), p["best"].get(sk)
+                if o is not None and int(sk) in part["splits"] and ("stream" if o[0][0] == 0 else "tile") in part["kinds"]:
+                    o = None   # re-measured: whatever the old entry says about this kind is out of date
+                cands = [c for c in (o, n) if c is not None]
+                if cands:
+                    best[sk] = min(cands, key=lambda c: c[1])
+            old["best"] = best
+            rows[key] = old
+            changed += 1
+    with open(args.main, "w") as f:
+        for key in sorted(rows):
+            f.write(json.dumps(rows[key]) + "\n")
+    print("%s: %d problems, %d partial rows folded in" % (args.main, len(rows), changed))
 
 
 def compact(args):
@@ -222,12 +270,18 @@ def main(argv=None):
     s.add_argument("--k", default="")
     s.add_argument("--n", default="")
     s.add_argument("--pairs", default="", help="OCxIC,OCxIC,... instead of the m x k grid, or `models` for the built-in list of layer shapes")
+    s.add_argument("--kinds", default="", help="stream, tile or both (comma-separated): measure only these kernels' shapes (the rows are partial: see merge)")
+    s.add_argument("--splits", default="", help="measure only these splitK values (the rows are partial: see merge)")
     s.add_argument("--iters", type=int, default=30)
     s.add_argument("--reps", type=int, default=5)
     s.set_defaults(fn=sweep)
     e = sub.add_parser("emit")
     e.add_argument("files", nargs="+")
     e.set_defaults(fn=emit)
+    m = sub.add_parser("merge")
+    m.add_argument("main")
+    m.add_argument("parts", nargs="+")
+    m.set_defaults(fn=merge)
     c = sub.add_parser("compact")
     c.add_argument("files", nargs="+")
     c.set_defaults(fn=compact)

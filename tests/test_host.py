@@ -196,11 +196,11 @@ def test_reference_heuristic_is_kept_verbatim():
 def test_mi355x_heuristic_prefers_no_split_when_rows_fill_the_chip():
     for (M, N, K) in [(4096, 8, 4096), (11008, 8, 4096), (8192, 16, 8192), (28672, 8, 8192), (8192, 512, 8192)]:
         assert fp6.heuristic_splitk_mi355x(M, N, K) == 1
-    # batches above 16 tile the rows in blocks of 64..256: K is cut to make up the missing parallelism, by a power of two
-    # of at most 8 and never into more pieces than there are 256-column K blocks
+    # batches above 16 tile the rows in blocks of 64..256: K is cut to make up the missing parallelism, into 2, 3, 4, 6 or 8
+    # pieces and never into more pieces than there are 256-column K blocks
     for (M, N, K) in [(8192, 32, 8192), (28672, 32, 8192), (8192, 64, 8192), (4096, 32, 11008), (10240, 32, 8192), (4096, 128, 512)]:
         s = fp6.heuristic_splitk_mi355x(M, N, K)
-        assert s in (1, 2, 4, 8) and s <= (K + 255) // 256, (M, N, K, s)
+        assert s in (1, 2, 3, 4, 6, 8) and s <= (K + 255) // 256, (M, N, K, s)
     assert fp6.heuristic_splitk_mi355x(8192, 32, 8192) > 1          # 64 row blocks alone leave three quarters of the CUs idle
     s = fp6.heuristic_splitk_mi355x(256, 8, 28672)      # 16 row tiles cannot occupy 256 CUs: splitting K pays
     assert 2 <= s <= 64
@@ -242,8 +242,8 @@ def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it()
                 continue
             assert v[:5] in compiled, (xb, OC, IC, BS, v)
             assert OC % tune.tile_rows(v[:5]) == 0
-            assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, 1 << i, shape) == 0
-            assert tuple(shape) == v[:5], (xb, OC, IC, BS, 1 << i, tuple(shape), v)
+            assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, tune.SPLITS[i], shape) == 0
+            assert tuple(shape) == v[:5], (xb, OC, IC, BS, tune.SPLITS[i], tuple(shape), v)
     # any legal problem gets a compiled shape that divides its rows, measured neighbour or not
     for (OC, IC, BS, sk) in [(256, 64, 1, 1), (768, 1088, 3, 2), (4352, 4160, 8, 1), (9984, 3008, 40, 3), (65536, 16384, 700, 1), (512, 64, 17, 1)]:
         for (E, Mb) in FORMATS:
@@ -497,7 +497,7 @@ def test_tuner_candidates_and_table_emission(tmp_path, monkeypatch):
     monkeypatch.setattr(tune, "INC_PATH", str(tmp_path / "out.inc"))
     tune.main(["emit", str(src)])
     lines = [l for l in (tmp_path / "out.inc").read_text().splitlines() if l.startswith("{")]
-    assert lines == ["{6,2,16,8,{{0,1,1,1,8,160},{255,0,0,0,0,0},{0,1,2,1,4,200},{255,0,0,0,0,0}}},"]
+    assert lines == ["{6,2,16,8,{{0,1,1,1,8,160},{255,0,0,0,0,0},{255,0,0,0,0,0},{0,1,2,1,4,200},{255,0,0,0,0,0},{255,0,0,0,0,0}}},"]
 
 
 # ------------------------------------------------------------------------------------------------ randomized round trips
