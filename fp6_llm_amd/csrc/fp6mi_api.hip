@@ -28,7 +28,8 @@ __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, con
     size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= MN) return;
     v4f sum = { 0.f, 0.f, 0.f, 0.f };
-    // eight, four or two loads in flight instead of one round trip to memory per split; the order of the sum is unchanged
+    // up to eight loads in flight instead of one round trip to memory per split; the order of the sum is unchanged.  The
+    // remainder after the groups of eight is one group of its exact size (a 3 done as 2 + 1 would be two round trips).
     auto chunk = [&](auto count, int s0) {
         constexpr int C = decltype(count)::value;
         v4f           part[C];
@@ -39,9 +40,16 @@ __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, con
     };
     int s = 0;
     for (; s + 8 <= splitK; s += 8) chunk(std::integral_constant<int, 8>{}, s);
-    if (s + 4 <= splitK) { chunk(std::integral_constant<int, 4>{}, s); s += 4; }
-    if (s + 2 <= splitK) { chunk(std::integral_constant<int, 2>{}, s); s += 2; }
-    if (s < splitK) chunk(std::integral_constant<int, 1>{}, s);
+    switch (splitK - s) {
+    case 7: chunk(std::integral_constant<int, 7>{}, s); break;
+    case 6: chunk(std::integral_constant<int, 6>{}, s); break;
+    case 5: chunk(std::integral_constant<int, 5>{}, s); break;
+    case 4: chunk(std::integral_constant<int, 4>{}, s); break;
+    case 3: chunk(std::integral_constant<int, 3>{}, s); break;
+    case 2: chunk(std::integral_constant<int, 2>{}, s); break;
+    case 1: chunk(std::integral_constant<int, 1>{}, s); break;
+    default: break;
+    }
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
     v4h o = { (half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3] };
     *reinterpret_cast<v4h *>(C + i) = o;

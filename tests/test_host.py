@@ -528,3 +528,15 @@ def test_packers_round_trip_on_random_shapes_and_bits():
 
     check()
 
+
+
+def test_host_code_and_oracle_are_clean_under_asan_and_ubsan():
+    """Builds tests/sanitize (the engine's CPU functions + the oracle with AddressSanitizer and UBSan, ROCm's clang) and runs its
+    driver over every format, cut K blocks, in-place packing and the grouped dequantizer."""
+    import shutil
+    import subprocess
+    d = os.path.join(os.path.dirname(os.path.abspath(__file__)), "sanitize")
+    if not os.path.exists("/opt/rocm/llvm/bin/clang++") or not shutil.which("make") or not os.path.isdir(d):
+        pytest.skip("needs ROCm's clang and make")
+    res = subprocess.run(["make", "-C", d, "-B", "run"], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0 and "clean under ASan + UBSan" in res.stdout, res.stdout[-2000:] + res.stderr[-2000:]
