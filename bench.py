@@ -474,6 +474,7 @@ def main():
                        with_system_blas=not args.no_cpu_baseline)
     E, M, OC, IC, BS = WORKLOADS[args.workload]
     res["lib_version"] = _lib.lib().fp6mi_version()
+    res["launch_table"] = _lib.lib().fp6mi_tuning_info().decode()
     if not (args.no_configs or args.calibrate_copy):
         res["configs"] = run_configs(device, args.configs_budget)
     compute_bound = BS >= 128

@@ -26,6 +26,7 @@ def lib():
     sigs = {
         "fp6mi_error_string": (ctypes.c_char_p, [ci]),
         "fp6mi_version": (ci, []),
+        "fp6mi_tuning_info": (ctypes.c_char_p, []),
         "fp6mi_prepack_ref": (ci, [ci, ci, vp, vp, sz, sz]),
         "fp6mi_dequant": (ci, [ci, ci, vp, vp, sz, sz, vp]),
         "fp6mi_unpack_ref": (ci, [ci, ci, vp, vp, sz, sz]),
@@ -63,7 +64,7 @@ def lib():
     return L
 
 
-EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_prepack_ref", "fp6mi_dequant", "fp6mi_unpack_ref",
+EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_tuning_info", "fp6mi_prepack_ref", "fp6mi_dequant", "fp6mi_unpack_ref",
             "fp6mi_native_bytes", "fp6mi_prepack_native", "fp6mi_relayout_ref_to_native", "fp6mi_unpack_native",
             "fp6mi_heuristic_splitk", "fp6mi_heuristic_splitk_format", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_twin_evict", "fp6mi_twin_clear",
             "fp6mi_linear_native_static", "fp6mi_static_workspace_bytes", "fp6mi_init",

@@ -305,6 +305,13 @@ const char *fp6mi_error_string(int code)
     }
 }
 
+const char *fp6mi_tuning_info(void)
+{
+    return
+#include "fp6mi_tuning_info.inc"
+        ;
+}
+
 int fp6mi_version(void) { return 130; } // 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }

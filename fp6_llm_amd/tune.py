@@ -108,6 +108,7 @@ class Bench:
         self.iters, self.reps, self.pool_bytes = iters, reps, pool_bytes
         self.dev = torch.device("cuda:0")
         self.key = None
+        self.lib_version, self.rocm = int(self.L.fp6mi_version()), str(torch.version.hip)   # stamped on every row measured
 
     def _pool(self, E, M, OC, IC):
         torch = self.torch
@@ -182,7 +183,7 @@ def sweep(args):
                         t = bench(E, M, OC, IC, BS, cfg, sk)
                         if t is not None and (str(sk) not in best or t < best[str(sk)][1]):
                             best[str(sk)] = [list(cfg), round(t, 3)]
-                    row = {"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best}
+                    row = {"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best, "lib": bench.lib_version, "rocm": bench.rocm}
                     if kinds or splits:   # a partial row: `merge` folds it into a full one
                         row["partial"] = {"kinds": sorted(kinds) if kinds else ["stream", "tile"], "splits": sorted(splits) if splits else list(SPLITS)}
                     f.write(json.dumps(row) + "\n")
@@ -197,7 +198,13 @@ def emit(args):
         for line in open(path):
             r = json.loads(line)
             rows[(1 + r["E"] + r["M"], r["BS"], r["OC"], r["IC"])] = r   # later files override earlier ones
+    stamps = {}
+    for r in rows.values():
+        key = "library version %s, ROCm %s" % (r["lib"], r["rocm"]) if "lib" in r else "unstamped (before rows carried a stamp)"
+        stamps[key] = stamps.get(key, 0) + 1
+    stamp_text = "; ".join("%d rows: %s" % (n, k) for k, n in sorted(stamps.items()))
     lines = ["// Measured launch shapes: generated by `python -m fp6_llm_amd.tune emit`; do not edit by hand.",
+             "// Measured on one MI355X (256 CUs). " + stamp_text,
              "// {bits, M/256, K/64, N, {best shape for splitK 1, 2, 3, 4, 6, 8: kind, n_tiles, row_tiles, row_waves, k_waves, time in 0.02 us}}"]
     for (xb, BS, OC, IC) in sorted(rows):
         r = rows[(xb, BS, OC, IC)]
@@ -211,6 +218,8 @@ def emit(args):
         lines.append("{%d,%d,%d,%d,{%s}}," % (xb, OC // 256, IC // 64, BS, ",".join(cells)))
     with open(INC_PATH, "w") as f:
         f.write("\n".join(lines) + "\n")
+    with open(INC_PATH.replace(".inc", "_info.inc"), "w") as f:   # the same stamp as a string the library can report
+        f.write('"%d entries; %s"\n' % (len(rows), stamp_text.replace('"', "'")))
     print("%d entries -> %s" % (len(rows), INC_PATH))
 
 
@@ -237,6 +246,9 @@ def merge(args):
                 if cands:
                     best[sk] = min(cands, key=lambda c: c[1])
             old["best"] = best
+            for stamp in ("lib", "rocm"):   # the row is as new as its newest part
+                if stamp in p:
+                    old[stamp] = p[stamp]
             rows[key] = old
             changed += 1
     with open(args.main, "w") as f:

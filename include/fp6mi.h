@@ -42,6 +42,10 @@ extern "C" {
 
 const char *fp6mi_error_string(int code);
 int         fp6mi_version(void);
+/* What the measured launch-shape table of this build was measured on: entry count, and per group of entries the library
+ * version and ROCm release of the measuring run.  The table answers only for 256-CU parts; elsewhere the rules decide.
+ * (No counterpart in the reference, whose tile choice is a fixed bucketing of the batch, fp6_llm/csrc/fp6_linear.cu:58-99.) */
+const char *fp6mi_tuning_info(void);
 
 /* ------------------------------------------------------------------------------------------------ CPU side */
 

@@ -16,7 +16,27 @@ import numpy as np
 import pytest
 
 import oracle
-from fp6_llm_amd import quant, synth
+
+# Inputs are made here, with nothing of the product in the way: the oracle is pinned before the product is compared with it.
+
+
+def _splitmix_codes(seed, OC, IC, E, M):
+    """The codes of the committed fixtures: element i = top x bits of splitmix64(seed + (i+1) * golden ratio)."""
+    mask = np.uint64(0xFFFFFFFFFFFFFFFF)
+    with np.errstate(over="ignore"):
+        z = (np.uint64(seed) + np.arange(1, OC * IC + 1, dtype=np.uint64) * np.uint64(0x9E3779B97F4A7C15)) & mask
+        z = ((z ^ (z >> np.uint64(30))) * np.uint64(0xBF58476D1CE4E5B9)) & mask
+        z = ((z ^ (z >> np.uint64(27))) * np.uint64(0x94D049BB133111EB)) & mask
+        z = z ^ (z >> np.uint64(31))
+    return (z >> np.uint64(64 - (1 + E + M))).astype(np.uint8).reshape(OC, IC)
+
+
+def _problem(seed, OC, IC, BS, E=3, M=2):
+    """Uniform random codes, scales in [1e-3, 1e-2], N(0,1) activations: (raw int32, scales, x)."""
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 1 << (1 + E + M), size=(OC, IC), dtype=np.uint8)
+    return (oracle.codes_to_raw(codes, E, M).view(np.int32), rng.uniform(1e-3, 1e-2, OC).astype(np.float16),
+            rng.standard_normal((BS, IC)).astype(np.float16))
 
 FORMATS = [(3, 2), (2, 2), (2, 3), (2, 1)]
 CODE_OF_ONE = {(3, 2): 0b001100, (2, 2): 0b00100, (2, 3): 0b001000, (2, 1): 0b0010}   # sign 0, exponent = bias, mantissa 0
@@ -67,14 +87,14 @@ def test_golden_prepack_fixtures(golden_dir):
         # the fixture's input is what the generator produces from its seed (fixtures are reproducible)
         OC = z["raw"].shape[0]
         IC = z["raw"].shape[1] * 32 // (1 + E + M)
-        assert (oracle.codes_to_raw(synth.uniform_codes(int(z["seed"]), OC, IC, E, M), E, M).view(np.int32) == z["raw"]).all()
+        assert (oracle.codes_to_raw(_splitmix_codes(int(z["seed"]), OC, IC, E, M), E, M).view(np.int32) == z["raw"]).all()
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_golden_hash_config1(golden_dir, E, M):
     name = "e%dm%d_256x1024_seed1001" % (E, M)
     ref = json.load(open(os.path.join(golden_dir, "prepack_hashes.json")))[name]
-    raw = oracle.codes_to_raw(synth.uniform_codes(1001, 256, 1024, E, M), E, M).view(np.int32)
+    raw = oracle.codes_to_raw(_splitmix_codes(1001, 256, 1024, E, M), E, M).view(np.int32)
     assert hashlib.sha256(raw.tobytes()).hexdigest() == ref["raw_sha256"]
     assert hashlib.sha256(oracle.prepack(raw, E, M).tobytes()).hexdigest() == ref["packed_sha256"]
 
@@ -261,7 +281,7 @@ def test_gemm_special_cases(E, M):
     out = oracle.gemm(wdq, np.ones((3, IC), np.float16))
     assert (out == np.float16(IC)).all()                     # all ones => every output = IC (kernel_test_fpx.py:98-99)
     # one-hot activations pick a column of the dequantized weights exactly
-    raw, sc, _ = synth.uniform_problem(3, OC, IC, 1, E, M)
+    raw, sc, _ = _problem(3, OC, IC, 1, E, M)
     wdq = oracle.dequant(raw, sc, E, M)
     x = np.zeros((2, IC), np.float16)
     x[0, 5] = 1
@@ -272,7 +292,7 @@ def test_gemm_special_cases(E, M):
 
 
 def test_gemm_against_float64_and_split_k():
-    raw, sc, x = synth.uniform_problem(11, 64, 256, 5)
+    raw, sc, x = _problem(11, 64, 256, 5)
     wdq = oracle.dequant(raw, sc)
     ref = oracle.gemm_f64(wdq, x)
     for s in (1, 2, 3, 4, 7):
