@@ -39,6 +39,7 @@ def lib():
         "fp6mi_workspace_bytes": (sz, [sz, sz, ci]),
         "fp6mi_linear_native": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci]),
         "fp6mi_linear": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci]),
+        "fp6mi_linear_stateless": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci, vp]),
         "fp6mi_linear_native_static": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz, sz, ci]),
         "fp6mi_static_workspace_bytes": (sz, []),
         "fp6mi_init": (ci, []),
@@ -66,7 +67,7 @@ def lib():
 
 EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_tuning_info", "fp6mi_prepack_ref", "fp6mi_dequant", "fp6mi_unpack_ref",
             "fp6mi_native_bytes", "fp6mi_prepack_native", "fp6mi_relayout_ref_to_native", "fp6mi_unpack_native",
-            "fp6mi_heuristic_splitk", "fp6mi_heuristic_splitk_format", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_twin_evict", "fp6mi_twin_clear",
+            "fp6mi_heuristic_splitk", "fp6mi_heuristic_splitk_format", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_linear_stateless", "fp6mi_twin_evict", "fp6mi_twin_clear",
             "fp6mi_linear_native_static", "fp6mi_static_workspace_bytes", "fp6mi_init",
             "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch",
             "fp6mi_group_exps_bytes", "fp6mi_pack_group_exps", "fp6mi_dequant_grouped", "fp6mi_linear_native_grouped",

@@ -543,6 +543,18 @@ int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc,
     return fp6mi_linear_native(E, Mb, stream, native, sc, B, C, M, N, K, ws, splitK);
 }
 
+int fp6mi_linear_stateless(int E, int Mb, void *stream, const void *W_ref, const void *sc, const void *B, void *C, size_t M, size_t N, size_t K,
+                           float *ws, int splitK, void *native_scratch)
+{
+    if (!native_scratch) return FP6MI_ERR_NULL;
+    if (!aligned16(native_scratch) || native_scratch == W_ref) return native_scratch == W_ref ? FP6MI_ERR_SHAPE : FP6MI_ERR_ALIGN;
+    int rc = check_gemm_args(E, Mb, W_ref, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native_scratch, W_ref, M, K);
+    if (rc != FP6MI_OK) return rc;
+    return fp6mi_linear_native(E, Mb, stream, native_scratch, sc, B, C, M, N, K, ws, splitK);
+}
+
 int fp6mi_twin_evict(const void *W_ref)
 {
     std::lock_guard<std::mutex> lock(g_twin_mutex);

@@ -118,6 +118,15 @@ int fp6mi_linear(int E, int Mbits, void *stream, const void *W_ref, const void *
 int fp6mi_twin_evict(const void *W_ref);
 int fp6mi_twin_clear(void);
 
+/* The same drop-in with the reference's contract kept to the letter (fp6_llm/csrc/fp6_linear.cu:104-139: the entry point
+ * allocates nothing and remembers nothing): W_ref is the REFERENCE layout, and the caller lends a device buffer of
+ * fp6mi_native_bytes(E, Mbits, M, K) bytes into which the weights are re-laid out on `stream` by every call, right before
+ * the GEMM reads them there.  No library state, safe under stream capture, any stream; the price is one more pass over the
+ * weights per call (read + write, about as long again as a batch-8 GEMM), so callers that can keep the converted copy
+ * should convert once (fp6mi_relayout_ref_to_native_gpu) and call fp6mi_linear_native. */
+int fp6mi_linear_stateless(int E, int Mbits, void *stream, const void *W_ref, const void *scales_f16, const void *B_f16,
+                           void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK, void *native_scratch);
+
 /* Tuning hook: the same GEMM with the launch shape chosen by the caller instead of the built-in selection
  * (no counterpart in the reference, whose TilingConfig is picked inside fpx_linear_kernel, fp6_linear.cu:61-81).
  * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup),

@@ -276,6 +276,49 @@ def test_c_abi_drop_in_second_stream_and_capture():
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
+def test_c_abi_stateless_drop_in_on_reference_layout(E, M):
+    """fp6mi_linear_stateless: reference-layout weights plus a caller-owned scratch buffer, nothing allocated and nothing kept
+    (the reference's contract, fp6_linear.cu:104-139).  Its first call may be a captured one; replays see weights that changed
+    in place between them; the result equals the explicit convert-then-GEMM route bit for bit."""
+    print("case stateless", E, M, flush=True)
+    L = _lib.lib()
+    OC, IC, N = 512, 1344, 11
+    raw, sc, x = synth.uniform_problem(730, OC, IC, N, E, M)
+    packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    out = torch.zeros((N, OC), dtype=torch.float16, device=DEV)
+    scratch = torch.empty(fp6.native_bytes(E, M, OC, IC), dtype=torch.uint8, device=DEV)
+    ws = torch.empty(2 * N * OC, dtype=torch.float32, device=DEV)
+    assert L.fp6mi_twin_clear() == 0
+
+    def call(stream, splitK):
+        return L.fp6mi_linear_stateless(E, M, stream.cuda_stream, packed.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), OC, N, IC,
+                                        ws.data_ptr(), splitK, scratch.data_ptr())
+    st = torch.cuda.Stream()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(st):
+        with torch.cuda.graph(g, stream=st):
+            assert call(st, 2) == 0                     # first use of these weights anywhere: inside a capture
+    g.replay()
+    torch.cuda.synchronize()
+    y_graph = out.cpu().numpy().copy()
+    check_close(y_graph, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "captured first call")
+    native = fp6.to_native(packed, E, M)
+    assert np.array_equal(y_graph.view(np.uint16), gemm_capi(E, M, native, scd, xd, OC, 2).view(np.uint16))
+    raw2, _, _ = synth.uniform_problem(731, OC, IC, N, E, M)
+    packed.copy_(fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw2)))   # new weights at the same address: no state to evict
+    g.replay()
+    torch.cuda.synchronize()
+    check_close(out.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw2, sc, E, M), x), "replay after the weights changed in place")
+    assert call(torch.cuda.current_stream(), 1) == 0
+    torch.cuda.synchronize()
+    check_close(out.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw2, sc, E, M), x), "eager call")
+    # argument errors: no scratch, scratch aliasing the weights
+    args = [E, M, None, packed.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), OC, N, IC, None, 1]
+    assert L.fp6mi_linear_stateless(*args, None) == -3 and L.fp6mi_linear_stateless(*args, packed.data_ptr()) == -2
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
 @pytest.mark.parametrize("N", [1, 3, 4, 5, 8, 9, 13, 16, 40])
 def test_infinite_activation_next_to_padded_columns(E, M, N):
     """K = 320 leaves 192 padding columns in the last 256-column block of the native layout.  An infinite activation in

@@ -540,3 +540,11 @@ def test_host_code_and_oracle_are_clean_under_asan_and_ubsan():
         pytest.skip("needs ROCm's clang and make")
     res = subprocess.run(["make", "-C", d, "-B", "run"], capture_output=True, text=True, timeout=600)
     assert res.returncode == 0 and "clean under ASan + UBSan" in res.stdout, res.stdout[-2000:] + res.stderr[-2000:]
+
+
+def test_the_reference_package_name_imports_the_same_functions():
+    """`import fp6_llm` (the reference's package name, fp6_llm/__init__.py:1) gives the engine's functions under the reference's names."""
+    import fp6_llm
+    for name in ["linear_forward_cuda", "weight_prepacking_cpu", "weight_dequant_cpu", "linear_forward_eXmY_cuda", "weight_prepacking_eXmY_cpu",
+                 "weight_dequant_eXmY_cpu", "Num_Wave", "HeuristicFuntion_SplitK"]:
+        assert getattr(fp6_llm, name) is getattr(fp6, name)
