@@ -591,30 +591,46 @@ __device__ __forceinline__ void tile_segment(v4f (&acc)[RT][NT], const uint8_t *
     }
 }
 
-// Scales the sums of one wavefront's RT x NT output tiles and stores them: fp16 into C, or fp32 partial sums into `part`
-// ([N][M] floats) when that is not null.  acc[r][t][i]: output row (R0+r)*16 + 4q+i, batch column nbase + 16t + col.
+// The tile kernel's output goes through LDS.  An MFMA accumulator holds four consecutive rows of ONE batch column per lane, so
+// a store straight from the accumulators makes the 16 lanes of a quarter-wavefront write 8 or 16 bytes into each of 16
+// different lines (C and the partial sums are [N][M], rows contiguous); the memory pipeline takes a line at a time, and with
+// every workgroup finishing at the same moment nothing hides it: measured, those stores were 10-16 % of the GEMMs that split K
+// at batches 32-128 and 4-5 % at batch 512.  So the wavefronts that hold results scale them and park them in LDS as a
+// [column][row] tile (fp16 for the final output, fp32 for partial sums), and after a barrier every thread of the workgroup
+// stores 16 consecutive bytes of one column: a wavefront writes whole lines.
+//   stage: TN columns of TM rows, column stride TM * (2 or 4) + 16 bytes
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
-template <int FM, int NT, int RT>
-__device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], half_t *__restrict__ C, float *__restrict__ part, uint32_t M,
-                                           uint32_t N, uint32_t R0, uint32_t nbase, int col, int q)
+template <int NT, int RT, int WR> constexpr size_t tile_stage_bytes(bool partial) { return (size_t)NT * 16 * (WR * RT * 16 * (partial ? 4 : 2) + 16); }
+
+template <int FM, int NT, int RT, int WR, int NTHREADS, typename OutT>
+__device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], OutT *__restrict__ out, uint8_t *stage, bool holds_results,
+                                           uint32_t M, uint32_t N, uint32_t mb, uint32_t nbase, int tid, int wr, int col, int q)
 {
+    constexpr int TM = WR * RT * 16, TN = NT * 16, kStride = TM * (int)sizeof(OutT) + 16, kPer16 = 16 / (int)sizeof(OutT); // outputs per 16 bytes
+    if (holds_results) {
 #pragma unroll
-    for (int r = 0; r < RT; r++) {
-        const uint32_t mg = (R0 + r) * 16 + 4 * q;
+        for (int r = 0; r < RT; r++)
 #pragma unroll
-        for (int t = 0; t < NT; t++) {
-            const uint32_t ng = nbase + 16 * t + col;
-            if (ng < N) {
+            for (int t = 0; t < NT; t++) {
                 v4f v;
 #pragma unroll
                 for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
-                if (!part) {
-                    v4h o = { (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
-                    *reinterpret_cast<v4h *>(C + (size_t)ng * M + mg) = o;
-                } else {
-                    *reinterpret_cast<v4f *>(part + (size_t)ng * M + mg) = v;
-                }
+                uint8_t *dst = stage + (16 * t + col) * kStride + ((wr * RT + r) * 16 + 4 * q) * (int)sizeof(OutT);
+                if constexpr (sizeof(OutT) == 2)
+                    *reinterpret_cast<v4h *>(dst) = (v4h){ (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
+                else
+                    *reinterpret_cast<v4f *>(dst) = v;
             }
+    }
+    __syncthreads();
+    constexpr int kPiecesPerCol = TM / kPer16, kPieces = TN * kPiecesPerCol;
+#pragma unroll
+    for (int p = tid; p < kPieces; p += NTHREADS) {
+        const int      c = p / kPiecesPerCol, piece = p % kPiecesPerCol;
+        const uint32_t ng = nbase + c;
+        if (ng < N) {
+            const v4u d = *reinterpret_cast<const v4u *>(stage + c * kStride + piece * 16);
+            *reinterpret_cast<v4u *>(out + (size_t)ng * M + (size_t)mb * TM + piece * kPer16) = d;
         }
     }
 }
@@ -658,7 +674,13 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
 
     tile_segment<FM, GS, NT, RT, WR, WK>(acc, W, gexp, X, N, K, units, mb, nbase, u0, u1, lds, tid, lane, wr, wk, col, q);
 
-    if (wk == 0) tile_store<FM, NT, RT>(acc, sc4, C, splitK == 1 ? nullptr : ws + (size_t)split * N * M, M, N, R0, nbase, col, q);
+    // the output tile is parked where the partial sums of the K wavefronts met: everybody has read those first
+    if (WK > 1) __syncthreads();
+    uint8_t *stage = lds;
+    if (splitK == 1)
+        tile_store<FM, NT, RT, WR, NTHREADS>(acc, sc4, C, stage, wk == 0, M, N, mb, nbase, tid, wr, col, q);
+    else
+        tile_store<FM, NT, RT, WR, NTHREADS>(acc, sc4, ws + (size_t)split * N * M, stage, wk == 0, M, N, mb, nbase, tid, wr, col, q);
 }
 
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
@@ -961,11 +983,13 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *gexp,
 {
     constexpr int TN = NT * 16, TM = WR * RT * 16;
     constexpr size_t x_bytes = 2 * (size_t)WK * TN * kXsRowBytes, red_bytes = WK > 1 ? (size_t)WK * WR * RT * NT * 1024 : 0;
-    constexpr size_t lds_bytes = x_bytes > red_bytes ? x_bytes : red_bytes;
-    static_assert(lds_bytes <= 160 * 1024, "tile does not fit in LDS");
+    constexpr size_t kLoopLds = x_bytes > red_bytes ? x_bytes : red_bytes, out_max = tile_stage_bytes<NT, RT, WR>(true);
+    constexpr size_t kMaxLds = kLoopLds > out_max ? kLoopLds : out_max;
+    static_assert(kMaxLds <= 160 * 1024, "tile does not fit in LDS");
+    const size_t out_bytes = tile_stage_bytes<NT, RT, WR>(splitK > 1), lds_bytes = kLoopLds > out_bytes ? kLoopLds : out_bytes;
     if (M % TM) return FP6MI_ERR_SHAPE;
-    if (lds_bytes > 48 * 1024)
-        if (int rc = allow_dynamic_lds<&gemm_tile<FM, GS, NT, RT, WR, WK>>(lds_bytes)) return rc;
+    if (kMaxLds > 48 * 1024)
+        if (int rc = allow_dynamic_lds<&gemm_tile<FM, GS, NT, RT, WR, WK>>(kMaxLds)) return rc;
     uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
     size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
     if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
