@@ -17,14 +17,20 @@ class FPxLinear(torch.nn.Module):
     """y = x @ dequant(W)^T (+ bias) with W held in the native gfx950 layout.  Weights are buffers, not parameters:
     the layer is inference-only, like the kernels."""
 
-    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None, dequant_above=None, group_scales=False):
+    # Batch size from which dequantize + FP16 library GEMM beats the mixed-input kernel on the MI355X, whatever the matrix: measured
+    # through this module at 4096^2, 8192^2, 28672x8192 and 8192x28672, the route wins by 5-25 % from 3072 rows up, ties at 2048, and
+    # loses below (at 1024 rows by 25-30 %).
+    PREFILL_CROSSOVER = 3072
+
+    def __init__(self, in_features, out_features, exponent=3, mantissa=2, bias=None, split_k=None, dequant_above="auto", group_scales=False):
         """group_scales: the layer also holds one exponent byte per row and 128 columns (factor 1 until weights are loaded).
         dequant_above: batch size from which forward() dequantizes the weights to a temporary fp16 matrix on the GPU and calls
         the FP16 library GEMM instead (prefill).  The mixed-input kernel wins while the GEMM is bound by weight bytes; from a
-        couple of thousand rows the FP16 library runs 1.3-1.4 PFLOP/s against its 0.9-1.0 (measured at 8192 x 8192), which
-        pays for the dequantization pass.  None (default) never does: the temporary costs 2 bytes per weight."""
+        few thousand rows the FP16 library runs 1.3-1.5 PFLOP/s against its 0.9-1.0, which pays for the dequantization pass
+        (about 30 us at 8192 x 8192).  "auto" (default) = PREFILL_CROSSOVER rows; None never does (the temporary costs 2 bytes
+        per weight for the duration of the call); an integer sets the threshold."""
         super().__init__()
-        self.dequant_above = dequant_above
+        self.dequant_above = self.PREFILL_CROSSOVER if dequant_above == "auto" else dequant_above
         if out_features % 256 or in_features % 64:
             raise ValueError("FPxLinear needs out_features %% 256 == 0 and in_features %% 64 == 0")
         self.in_features, self.out_features = in_features, out_features

@@ -543,6 +543,7 @@ def test_module_prefill_route_dequantizes_and_matches():
     w = torch.from_numpy(synth.normal(53, (256, 512))).half()
     for (E, M) in FORMATS:
         layer = module.FPxLinear.from_float(w, E, M).to(DEV)
+        assert layer.dequant_above == module.FPxLinear.PREFILL_CROSSOVER == 3072   # the default: the measured crossover
         layer.dequant_above = 64
         x = torch.from_numpy(synth.activations(54, 100, 512)).to(DEV)
         y_lib = layer(x)                       # 100 rows >= 64: dequantize + FP16 library GEMM
