@@ -50,6 +50,7 @@ def lib():
         "fp6mi_dequant_native_gpu": (ci, [ci, ci, vp, vp, vp, vp, sz, sz]),
         "fp6mi_quantize_native_gpu": (ci, [ci, ci, vp, vp, vp, vp, ci, sz, sz]),
         "fp6mi_query_launch": (ci, [ci, ci, sz, sz, sz, ci, ctypes.POINTER(ci)]),
+        "fp6mi_launch_source": (ci, [ci, ci, sz, sz, sz, ci]),
         "fp6mi_group_exps_bytes": (sz, [sz, sz]),
         "fp6mi_pack_group_exps": (ci, [vp, vp, sz, sz]),
         "fp6mi_dequant_grouped": (ci, [ci, ci, vp, vp, sz, sz, vp, vp]),
@@ -69,7 +70,7 @@ EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_tuning_info", "fp6mi_p
             "fp6mi_native_bytes", "fp6mi_prepack_native", "fp6mi_relayout_ref_to_native", "fp6mi_unpack_native",
             "fp6mi_heuristic_splitk", "fp6mi_heuristic_splitk_format", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_linear_stateless", "fp6mi_twin_evict", "fp6mi_twin_clear",
             "fp6mi_linear_native_static", "fp6mi_static_workspace_bytes", "fp6mi_init",
-            "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch",
+            "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch", "fp6mi_launch_source",
             "fp6mi_group_exps_bytes", "fp6mi_pack_group_exps", "fp6mi_dequant_grouped", "fp6mi_linear_native_grouped",
             "fp6mi_dequant_native_grouped_gpu", "fp6mi_quantize_native_grouped_gpu"]
 

@@ -133,7 +133,7 @@ inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (
 // 16384 and 17920 rows differ by 9 % in size but by a whole round of 64-row workgroups; sweeps off the grid showed that
 // this, not the distance, decides which neighbour's shape is right.  Farther neighbours pay 15 % per octave of distance.
 struct TuneGroup { int xb; size_t n, begin, end; }; // entries [begin, end) of kTune share format and batch (the table is sorted by them)
-struct TuneAnswer { bool valid; LaunchCfg cfg[kNumSplits]; float t[kNumSplits]; }; // index i: splitK = kSplits[i]; t in 0.02 us, 0 = no proposal
+struct TuneAnswer { bool valid, measured; LaunchCfg cfg[kNumSplits]; float t[kNumSplits]; }; // index i: splitK = kSplits[i]; t in 0.02 us, 0 = no proposal; measured: this very (M, K) at this or the next larger measured batch
 
 const std::vector<TuneGroup> &tune_groups()
 {
@@ -191,7 +191,7 @@ const TuneAnswer *tune_lookup(int xbits, size_t M, size_t N, size_t K)
         }
     }
     TuneAnswer a = {};
-    if (count > 0 && dist[0] == 0.f) count = 1; // measured: nothing to carry over
+    if (count > 0 && dist[0] == 0.f) count = 1, a.measured = true; // measured: nothing to carry over
     const size_t units = (K + 255) / 256;
     for (int j = 0; j < count; j++) {
         const TuneEntry &e = *near[j];
@@ -432,6 +432,18 @@ int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const vo
     LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
     return linear_native(*fp6mi::ops_for(E, Mb), st, W, sc, nullptr, B, C, M, N, K, ws, splitK, &c);
+}
+
+int fp6mi_launch_source(int E, int Mb, size_t M, size_t N, size_t K, int splitK)
+{
+    if (!fp6mi::supported(E, Mb)) return FP6MI_ERR_FORMAT;
+    if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
+    if (splitK < 1) return FP6MI_ERR_SPLITK;
+    const int i = split_index(splitK);
+    if (i >= 0)
+        if (const TuneAnswer *a = tune_lookup(1 + E + Mb, M, N, K))
+            if (a->t[i] > 0.f) return a->measured ? 0 : 1;
+    return 2;
 }
 
 int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, int *shape)

@@ -143,6 +143,10 @@ int fp6mi_linear_native_cfg(int E, int Mbits, void *stream, const void *W_native
  * one, else from a rule; it plays the part of the reference's compile-time TilingConfig dispatch
  * (fp6_llm/csrc/fp6_linear.cu:61-81). */
 int fp6mi_query_launch(int E, int Mbits, size_t M, size_t N, size_t K, int splitK, int *shape);
+/* Where that choice comes from on a 256-CU part: 0 = this (M, K) was measured (at this batch or the next larger measured
+ * one), 1 = carried over from measured problems up to a factor 1.5 away in M and in K, 2 = the rules (no measured
+ * neighbour, or a splitK the table does not hold).  Negative: FP6MI_ERR_*.  (No counterpart in the reference.) */
+int fp6mi_launch_source(int E, int Mbits, size_t M, size_t N, size_t K, int splitK);
 
 /* Device-side conversion reference layout -> native layout (both device pointers), run once per weight matrix. */
 int fp6mi_relayout_ref_to_native_gpu(int E, int Mbits, void *stream, void *native_dev, const void *packed_ref_dev,

@@ -548,3 +548,14 @@ def test_the_reference_package_name_imports_the_same_functions():
     for name in ["linear_forward_cuda", "weight_prepacking_cpu", "weight_dequant_cpu", "linear_forward_eXmY_cuda", "weight_prepacking_eXmY_cpu",
                  "weight_dequant_eXmY_cpu", "Num_Wave", "HeuristicFuntion_SplitK"]:
         assert getattr(fp6_llm, name) is getattr(fp6, name)
+
+
+def test_launch_source_tells_measured_from_carried_over_from_rules():
+    L = _lib.lib()
+    assert L.fp6mi_launch_source(3, 2, 4096, 8, 4096, 1) == 0          # in the table
+    assert L.fp6mi_launch_source(3, 2, 4096, 7, 4096, 1) == 0          # the next larger measured batch of a measured matrix
+    assert L.fp6mi_launch_source(3, 2, 4352, 8, 4160, 1) == 1          # neighbours within a factor 1.5
+    assert L.fp6mi_launch_source(3, 2, 256, 8, 64, 1) == 2               # far from every measured problem
+    assert L.fp6mi_launch_source(3, 2, 4096, 8, 4096, 5) == 2          # a split the table does not hold
+    assert L.fp6mi_launch_source(4, 3, 4096, 8, 4096, 1) == -1 and L.fp6mi_launch_source(3, 2, 100, 8, 4096, 1) == -2
+    assert b"library version" in L.fp6mi_tuning_info()
