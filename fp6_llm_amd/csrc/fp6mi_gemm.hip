@@ -172,9 +172,11 @@ template <int FM, bool GS> __device__ __forceinline__ void convert(const WFrag<F
 // The vector memory pipeline looks up one line per cycle: measured on the MI355X with nothing else in the kernel, the
 // operand-order loads of a 4096-wide K for batch 16 on all 256 CUs take 3.1 us, the same bytes loaded as whole rows
 // (32 consecutive lanes = 512 consecutive bytes) 0.9 us; batch 8 with two MFMA steps per load 1.4 us against 0.25 us.
-// So every wavefront loads its slice as whole rows, writes it to an LDS area of its own (no barrier: nobody else reads it)
-// and reads it back in operand order; LDS rows are padded to 544 bytes, the stride at which that read is conflict-free.
-// Batches of at most 8 stage 8 rows (B columns 8..15 re-read rows 0..7 and feed outputs that are never stored).
+// So from batch 5 up every wavefront loads its slice as whole rows, writes it to an LDS area of its own (no barrier: nobody
+// else reads it) and reads it back in operand order; LDS rows are padded to 544 bytes, the stride at which that read is
+// conflict-free.  Batches of 5 to 8 stage 8 rows (B columns 8..15 re-read rows 0..7 and feed outputs that are never stored).
+// Batches up to 4 keep operand-order loads: a quarter-wavefront then touches at most 4 lines, and the trip through LDS
+// would only add latency (measured: 1-4 % slower there).
 // ---------------------------------------------------------------------------------------------------------------
 constexpr int kXsRowBytes = 544;
 
