@@ -22,11 +22,9 @@ typedef float    v4f __attribute__((ext_vector_type(4)));
 
 using fp6mi::LaunchCfg;
 
-// C[i] = fp16_rn(sum over splits, in split order, of ws[s][i]); four outputs per thread.
-__global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK)
+// C[i] = fp16_rn(sum over splits, in split order, of ws[s][i]) for the four outputs from index i.
+__device__ __forceinline__ void reduce_four(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK, size_t i)
 {
-    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= MN) return;
     v4f sum = { 0.f, 0.f, 0.f, 0.f };
     // up to eight loads in flight instead of one round trip to memory per split; the order of the sum is unchanged.  The
     // remainder after the groups of eight is one group of its exact size (a 3 done as 2 + 1 would be two round trips).
@@ -53,6 +51,32 @@ __global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, con
     typedef _Float16 v4h __attribute__((ext_vector_type(4)));
     v4h o = { (half_t)sum[0], (half_t)sum[1], (half_t)sum[2], (half_t)sum[3] };
     *reinterpret_cast<v4h *>(C + i) = o;
+}
+
+// four outputs per thread, in the order of the output
+__global__ __launch_bounds__(256) void splitk_reduce(half_t *__restrict__ C, const float *__restrict__ ws, size_t MN, int splitK)
+{
+    const size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i < MN) reduce_four(C, ws, MN, splitK, i);
+}
+
+// The same sums with the workgroups placed where the partial sums were written.  gemm_tile hands XCD x (workgroup ids
+// congruent to x mod 8) the consecutive (row block, split, column block) triples from start(x) = x * q + min(x, r) on, where
+// q = grid / 8 and r = grid mod 8, i.e. the row blocks from start(x) / per_block (per_block = splits x column blocks; a row block
+// cut by the boundary counts for the later XCD).  Workgroup b of this kernel also runs on XCD b mod 8 and takes the rows that
+// XCD produced, for every batch column: its loads hit the L2 that the partial sums were written through, where the
+// output-order kernel above finds most of them behind another XCD's L2 (measured: 4 MB written by one kernel are read by
+// the next in 0.7 us from the writer's XCD and in 2.6 us from another).
+__global__ __launch_bounds__(256) void splitk_reduce_by_xcd(half_t *__restrict__ C, const float *__restrict__ ws, uint32_t M, uint32_t N, int splitK,
+                                                             uint32_t tile_rows, uint32_t q, uint32_t r, uint32_t per_block)
+{
+    const uint32_t x = blockIdx.x & 7u, j = blockIdx.x >> 3;
+    const uint32_t s0 = x * q + (x < r ? x : r), s1 = (x + 1) * q + (x + 1 < r ? x + 1 : r);
+    const uint32_t lo = s0 / per_block * tile_rows, hi = s1 / per_block * tile_rows, quads = (hi - lo) / 4;
+    const uint32_t g = j * 256 + threadIdx.x;
+    if (g >= quads * N) return;
+    const uint32_t n = g / quads, m = lo + (g - n * quads) * 4;
+    reduce_four(C, ws, (size_t)M * N, splitK, (size_t)n * M + m);
 }
 
 inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
@@ -276,8 +300,23 @@ int linear_native(const fp6mi::FormatOps &ops, hipStream_t st, const void *W, co
     if (rc != 0) return rc;
     if (splitK > 1) {
         size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
-        hipLaunchKernelGGL(splitk_reduce, dim3((uint32_t)((MN / 4 + 255) / 256)), dim3(256), 0, st, static_cast<half_t *>(C), ws, MN,
-                           splitK);
+        const size_t tile_rows = (size_t)c.wr * c.rt * 16, nblocks = (N + (size_t)c.nt * 16 - 1) / ((size_t)c.nt * 16);
+        const size_t grid = c.kind == 1 && M % tile_rows == 0 ? M / tile_rows * nblocks * splitK : 0;
+        if (grid && MN / 4 < ((size_t)1 << 31)) {
+            // gemm_tile gave every XCD a run of consecutive triples: reduce where the partial sums lie
+            const uint32_t q = (uint32_t)(grid / 8), r = (uint32_t)(grid % 8), per_block = (uint32_t)(nblocks * splitK);
+            size_t         most = 0;
+            for (uint32_t x = 0; x < 8; x++) {
+                const size_t s0 = (size_t)x * q + (x < r ? x : r), s1 = (size_t)(x + 1) * q + (x + 1 < r ? x + 1 : r);
+                const size_t rows = (s1 / per_block - s0 / per_block) * tile_rows;
+                most = rows > most ? rows : most;
+            }
+            const size_t per_xcd = (most / 4 * N + 255) / 256;
+            hipLaunchKernelGGL(splitk_reduce_by_xcd, dim3((uint32_t)(per_xcd * 8)), dim3(256), 0, st, static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N,
+                               splitK, (uint32_t)tile_rows, q, r, per_block);
+        } else {
+            hipLaunchKernelGGL(splitk_reduce, dim3((uint32_t)((MN / 4 + 255) / 256)), dim3(256), 0, st, static_cast<half_t *>(C), ws, MN, splitK);
+        }
         rc = (int)hipGetLastError();
     }
     return rc;
@@ -312,7 +351,7 @@ const char *fp6mi_tuning_info(void)
         ;
 }
 
-int fp6mi_version(void) { return 131; } // 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
+int fp6mi_version(void) { return 132; } // 132: split-K reduction runs on the XCD that wrote the partial sums, every grid size gets XCD-contiguous tiles; 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
 int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }

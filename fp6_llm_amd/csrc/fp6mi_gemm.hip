@@ -653,10 +653,14 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     const int wr = wave % WR, wk = wave / WR;
     const int col = lane & 15, q = lane >> 4;
 
-    // grid.x -> (row block, column block, split): ids that are congruent mod 8 run on one XCD and share its L2, so
-    // the column blocks of a row block (which read the same weights) are given such ids
+    // grid.x -> (row block, split, column block): workgroup ids that are congruent mod 8 run on one XCD and share its L2, so
+    // XCD x is given a run of consecutive triples (the column blocks of a row block read the same weights, its splits write
+    // partial sums that one reduction workgroup reads): the first (gridDim.x mod 8) XCDs take one triple more than the others
     uint32_t id = blockIdx.x;
-    if ((gridDim.x & 7u) == 0) id = (id & 7u) * (gridDim.x >> 3) + (id >> 3);
+    {
+        const uint32_t q = gridDim.x >> 3, r = gridDim.x & 7u, x = id & 7u;
+        id = x * q + (x < r ? x : r) + (id >> 3);
+    }
     const uint32_t nb = id % nblocks, rest = id / nblocks, split = rest % splitK, mb = rest / splitK;
     const uint32_t nbase = nb * TN, R0 = (mb * WR + wr) * RT; // first row tile of this wavefront
 
