@@ -146,6 +146,31 @@ def test_every_launch_shape(E, M, cfg):
         check_close(gemm_capi(E, M, native, scd, xd, OC, splitK, cfg), ref, "cfg %s splitK %d" % (cfg, splitK))
 
 
+@pytest.mark.parametrize("OC,cfg,N,splitK", [
+    (256, (1, 2, 1, 4, 4), 17, 3),     # 4 row blocks x 3 splits = 12 workgroups: four XCDs get two triples, four get one
+    (768, (1, 2, 2, 4, 1), 40, 5),     # 6 row blocks x 5 splits x 2 column blocks = 60: XCD boundaries cut row blocks
+    (1280, (1, 4, 2, 8, 1), 70, 2),    # 5 row blocks of 256 rows x 2 x 2 = 20
+    (2816, (1, 2, 2, 4, 2), 33, 3),    # 22 row blocks x 3 x 2 = 132
+    (512, (1, 2, 2, 4, 1), 5, 2),      # 4 x 2 = 8: one triple per XCD, half the XCDs own no row block
+    (256, (1, 4, 2, 8, 1), 64, 6),     # one row block, six splits: a single XCD owns every row
+])
+def test_split_k_reduction_owns_every_row_once_on_any_grid(OC, cfg, N, splitK):
+    """The reduction behind the tile kernel deals the rows out by the XCD that wrote their partial sums; whatever the grid size
+    (multiple of 8 or not, fewer triples than XCDs, boundaries inside a row block) every output must be summed exactly once.
+    The output buffer starts as NaN, so a row nobody owned would show."""
+    print("case reduction ownership", OC, cfg, N, splitK, flush=True)
+    E, M, IC = 3, 2, 2304
+    raw, sc, x = synth.uniform_problem(900 + OC + N, OC, IC, N, E, M)
+    native, scd, xd = upload(raw, sc, x, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    y = gemm_capi(E, M, native, scd, xd, OC, splitK, cfg)
+    assert np.isfinite(y).all()
+    check_close(y, ref, "cfg %s splitK %d" % (cfg, splitK))
+    if N <= 16:  # the output-order reduction behind the small-batch kernel on the same problem
+        y_stream = gemm_capi(E, M, native, scd, xd, OC, splitK, (0, 1, 1, 1, 4))
+        check_close(y_stream, ref, "stream splitK %d" % splitK)
+
+
 def test_unsupported_launch_shape_is_rejected():
     raw, sc, x = synth.uniform_problem(1, 256, 256, 4)
     native, scd, xd = upload(raw, sc, x, 3, 2)
