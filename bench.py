@@ -197,6 +197,31 @@ def read_floor_us(prob, steps, warmup):
     return _capture_and_time(step, steps, warmup)[1]
 
 
+def xcd_locality_probe(device):
+    """Pairs of kernels in the benchmark's back-to-back graph: the first writes `wgs` regions, the second reads them, region
+    (b + shift) mod wgs by workgroup b.  Workgroup ids congruent mod 8 share an XCD, so shift 0 and 8 read through the L2 the
+    data was written through, shift 1 and 3 from another XCD.  Returns microseconds per pair, launches included."""
+    import ctypes
+
+    import torch
+
+    lib = ctypes.CDLL(os.path.join(ROOT, "fp6_llm_amd", "libfp6mi_probe.so"))
+    lib.fp6mi_probe_write_then_read.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_uint, ctypes.c_uint, ctypes.c_uint, ctypes.c_void_p]
+    lib.fp6mi_probe_write_then_read.restype = ctypes.c_int
+    buf = torch.empty(256 << 20, dtype=torch.uint8, device=device)
+    sink = torch.zeros(16, dtype=torch.int32, device=device)
+    rows = []
+    for wgs, per in ((256, 4), (256, 16), (256, 64), (512, 8)):
+        row = {"megabytes": round(wgs * per * 4096 / 1e6, 2), "workgroups": wgs}
+        for shift in (0, 8, 1, 3):
+            def step(i):
+                rc = lib.fp6mi_probe_write_then_read(torch.cuda.current_stream().cuda_stream, buf.data_ptr(), wgs, per, shift, sink.data_ptr())
+                assert rc == 0, rc
+            row["shift_%d_%s_xcd_us" % (shift, "same" if shift % 8 == 0 else "other")] = round(_capture_and_time(step, 100, 5)[1], 3)
+        rows.append(row)
+    return {"probe": "write kernel then read kernel, us per pair in a back-to-back graph", "rows": rows}
+
+
 class _RocblasFp16:
     """rocblas_gemm_ex (FP16 in/out, FP32 accumulation) through ctypes: the second FP16 library path on this stack, which
     for some shapes picks a faster kernel than torch's F.linear and for others a much slower one."""
@@ -451,6 +476,9 @@ def main():
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by; "
                          "skips the FP16, CPU and per-configuration legs")
+    ap.add_argument("--probe-xcd-locality", action="store_true",
+                    help="measurement aid: instead of the benchmark, time a write kernel followed by a read kernel whose workgroups run on "
+                         "the writer's XCD or on another one, and print the pair times")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         sys.exit("bench.py: this path runs on ONE GPU (a linear layer shards by output rows without any collective); use --gpus 1")
@@ -464,6 +492,9 @@ def main():
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
 
+    if args.probe_xcd_locality:
+        print(json.dumps(xcd_locality_probe(device)))
+        return
     if args.calibrate_copy:
         src = torch.empty(64 << 20, dtype=torch.uint8, device=device).random_()
         dst = torch.empty_like(src)
