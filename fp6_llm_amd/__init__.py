@@ -18,6 +18,7 @@ memory and streams.  Where the reference aborts the process (assert / exit) thes
 """
 import math
 import os
+import threading
 import weakref
 
 import torch
@@ -268,6 +269,7 @@ def weight_quantize_native_cuda(EXPONENT, MANTISSA, weight, group_scales=False):
 # ----------------------------------------------------------------------------------------------------------------
 _workspaces = {}   # (device index, stream) -> float32 tensor, grown on demand
 _native_cache = {}  # id(tensor) -> (weakref, version, data_ptr, E, M, native tensor)
+_native_cache_lock = threading.RLock()  # (re-entrant: a weak reference's callback may fire while the lock is held)
 
 
 def clear_caches():
@@ -352,17 +354,22 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
 
 def _native_of(weights, E, M):
     """Native-layout twin of a reference-layout GPU tensor, converted once and remembered while the tensor is alive
-    and unmodified (tensor identity, storage address and in-place version counter must all match)."""
+    and unmodified (tensor identity, storage address and in-place version counter must all match).  The twin is published
+    only once it is completely written: the one-time conversion waits for its kernel (unless the stream is being captured,
+    where the conversion becomes part of the graph), so a later call on any stream or thread may use it without further ordering."""
     key = id(weights)
-    hit = _native_cache.get(key)
-    if hit is not None:
-        ref, version, ptr, e, m, native = hit
-        if ref() is weights and version == weights._version and ptr == weights.data_ptr() and (e, m) == (E, M):
-            return native
-    native = to_native(weights, E, M)
-    _native_cache[key] = (weakref.ref(weights, lambda _r, k=key: _native_cache.pop(k, None)), weights._version,
-                          weights.data_ptr(), E, M, native)
-    return native
+    with _native_cache_lock:
+        hit = _native_cache.get(key)
+        if hit is not None:
+            ref, version, ptr, e, m, native = hit
+            if ref() is weights and version == weights._version and ptr == weights.data_ptr() and (e, m) == (E, M):
+                return native
+        native = to_native(weights, E, M)
+        if weights.device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
+            torch.cuda.current_stream(weights.device).synchronize()
+        _native_cache[key] = (weakref.ref(weights, lambda _r, k=key: _native_cache.pop(k, None)), weights._version,
+                              weights.data_ptr(), E, M, native)
+        return native
 
 
 def _sort_forward_args(a, b, c):

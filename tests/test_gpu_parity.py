@@ -300,6 +300,48 @@ def test_c_abi_drop_in_second_stream_and_capture():
     assert L.fp6mi_twin_clear() == 0
 
 
+def test_python_drop_in_twin_across_streams_and_threads():
+    """linear_forward_cuda keeps a native twin per reference-layout tensor.  The first call (which converts) runs on one stream,
+    the next at once on another, and two threads race for the first use of a second tensor: every result must be right."""
+    import threading
+
+    E, M, OC, IC, N = 3, 2, 2048, 4096, 8
+    raw, sc, x = synth.uniform_problem(720, OC, IC, N, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    packed = fp6.weight_prepacking_cpu(torch.from_numpy(raw)).to(DEV)
+    torch.cuda.synchronize()
+    sa, sb = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(sa):
+        ya = fp6.linear_forward_cuda(xd, packed, scd, 1)
+    with torch.cuda.stream(sb):
+        yb = fp6.linear_forward_cuda(xd, packed, scd, 1)
+    torch.cuda.synchronize()
+    check_close(ya.cpu().numpy(), ref, "first call, stream A")
+    check_close(yb.cpu().numpy(), ref, "second call, stream B")
+
+    packed2 = fp6.weight_prepacking_cpu(torch.from_numpy(raw)).to(DEV)
+    torch.cuda.synchronize()
+    results, errors = [None, None], []
+
+    def worker(k):
+        try:
+            with torch.cuda.stream(torch.cuda.Stream()):
+                results[k] = fp6.linear_forward_cuda(xd, packed2, scd, 1)
+        except Exception as exc:  # noqa: BLE001 (reported below)
+            errors.append(exc)
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for k in range(2):
+        check_close(results[k].cpu().numpy(), ref, "thread %d" % k)
+
+
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_c_abi_stateless_drop_in_on_reference_layout(E, M):
     """fp6mi_linear_stateless: reference-layout weights plus a caller-owned scratch buffer, nothing allocated and nothing kept
