@@ -355,8 +355,10 @@ def linear_forward_native(EXPONENT, MANTISSA, in_feats, native_weight, scales, O
 def _native_of(weights, E, M):
     """Native-layout twin of a reference-layout GPU tensor, converted once and remembered while the tensor is alive
     and unmodified (tensor identity, storage address and in-place version counter must all match).  The twin is published
-    only once it is completely written: the one-time conversion waits for its kernel (unless the stream is being captured,
-    where the conversion becomes part of the graph), so a later call on any stream or thread may use it without further ordering."""
+    only once it is completely written: the one-time conversion waits for its kernel, so a later call on any stream or thread
+    may use it without further ordering.  A first use while the current stream is being captured publishes nothing: there the
+    conversion is only recorded, its result lives in the graph's memory pool and is written by every replay, so the captured
+    GEMM gets a twin of its own and an eager call before the first replay converts for itself."""
     key = id(weights)
     with _native_cache_lock:
         hit = _native_cache.get(key)
@@ -364,8 +366,11 @@ def _native_of(weights, E, M):
             ref, version, ptr, e, m, native = hit
             if ref() is weights and version == weights._version and ptr == weights.data_ptr() and (e, m) == (E, M):
                 return native
+        capturing = weights.device.type == "cuda" and torch.cuda.is_current_stream_capturing()
         native = to_native(weights, E, M)
-        if weights.device.type == "cuda" and not torch.cuda.is_current_stream_capturing():
+        if capturing:
+            return native
+        if weights.device.type == "cuda":
             torch.cuda.current_stream(weights.device).synchronize()
         _native_cache[key] = (weakref.ref(weights, lambda _r, k=key: _native_cache.pop(k, None)), weights._version,
                               weights.data_ptr(), E, M, native)

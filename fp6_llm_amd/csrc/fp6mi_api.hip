@@ -337,7 +337,7 @@ const char *fp6mi_error_string(int code)
     case FP6MI_ERR_NULL: return "a required pointer is NULL";
     case FP6MI_ERR_WORKSPACE: return "splitK > 1 needs a workspace of splitK*M*N floats";
     case FP6MI_ERR_SPLITK: return "splitK must be >= 1";
-    case FP6MI_ERR_ALIGN: return "device pointers must be 16-byte aligned (scales: 8-byte)";
+    case FP6MI_ERR_ALIGN: return "weights, activations, output and workspace must be 16-byte aligned (scales: 2-byte, group exponents: 2-byte)";
     case FP6MI_ERR_TOO_LARGE: return "splitK*M*N floats exceed the library's static workspace (fp6mi_static_workspace_bytes)";
     case FP6MI_ERR_CAPTURE: return "the stream is being captured and this call would have to allocate: convert the weights first (fp6mi_relayout_ref_to_native_gpu) or make the first call outside the capture";
     default: return code > 0 ? hipGetErrorString((hipError_t)code) : "unknown fp6mi error";
@@ -439,7 +439,7 @@ static int check_gemm_args(int E, int Mb, const void *W, const void *sc, const v
     if (splitK < 1 || splitK > 65535) return FP6MI_ERR_SPLITK;
     if (splitK > 1 && !ws) return FP6MI_ERR_WORKSPACE;
     if (!aligned16(W) || !aligned16(B) || !aligned16(C) || (ws && !aligned16(ws))) return FP6MI_ERR_ALIGN;
-    if (reinterpret_cast<uintptr_t>(sc) & 7u) return FP6MI_ERR_ALIGN; // the tile kernel reads four row scales with one 8-byte load
+    if (reinterpret_cast<uintptr_t>(sc) & 1u) return FP6MI_ERR_ALIGN; // halfs; the tile kernel uses 8-byte loads where the pointer allows them
     return FP6MI_OK;
 }
 
@@ -491,7 +491,7 @@ int fp6mi_query_launch(int E, int Mb, size_t M, size_t N, size_t K, int splitK, 
     if (!shape) return FP6MI_ERR_NULL;
     if (M == 0 || M % 256 || K == 0 || K % 64 || N == 0) return FP6MI_ERR_SHAPE;
     if (splitK < 1) return FP6MI_ERR_SPLITK;
-    LaunchCfg c = pick_cfg(1 + E + Mb, M, N, K, splitK, 256);
+    LaunchCfg c = pick_cfg(1 + E + Mb, M, N, K, splitK, current_device_cus()); // the count the launch path uses (256 where no device answers)
     shape[0] = c.kind, shape[1] = c.nt, shape[2] = c.rt, shape[3] = c.wr, shape[4] = c.wk;
     return FP6MI_OK;
 }
@@ -559,7 +559,7 @@ int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc,
     if (rc != FP6MI_OK) return rc;
     int device = 0;
     if (hipError_t e = hipGetDevice(&device); e != hipSuccess) return (int)e;
-    void *native = nullptr;
+    void *native = nullptr, *stale = nullptr;
     {
         std::lock_guard<std::mutex> lock(g_twin_mutex);
         auto it = g_twins.find(W_ref);
@@ -568,28 +568,46 @@ int fp6mi_linear(int E, int Mb, void *stream, const void *W_ref, const void *sc,
             if (t.E == E && t.Mb == Mb && t.M == M && t.K == K && t.device == device) {
                 native = t.native;
             } else { // the address now holds a different matrix
-                (void)hipFree(t.native);
+                stale = t.native;
                 g_twins.erase(it);
             }
         }
-        if (!native) {
-            // A twin has to be allocated and filled: not possible while the stream is being captured (the allocation would end
-            // the capture with an error, and a replay would not repeat it).
-            hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-            if (hipError_t e = hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cap); e != hipSuccess) return (int)e;
-            if (cap != hipStreamCaptureStatusNone) return FP6MI_ERR_CAPTURE;
-            size_t bytes = fp6mi::native_bytes(E, Mb, M, K);
-            if (hipError_t e = hipMalloc(&native, bytes); e != hipSuccess) return (int)e;
-            rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K);
-            // The twin becomes visible to other callers (and other streams) only once it is completely written: this
-            // one-time path waits for the relayout kernel before it publishes the pointer.
-            if (rc == 0) rc = (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
-            if (rc != 0) {
-                (void)hipFree(native);
-                return rc;
-            }
-            g_twins[W_ref] = Twin{ native, E, Mb, M, K, device };
+    }
+    // Everything slow happens outside the lock (allocation, the relayout kernel, the wait for it, freeing a stale twin), so
+    // that other threads' calls, cache hits on other weights above all, never queue behind one caller's stream.
+    if (stale) (void)hipFree(stale);
+    if (!native) {
+        // A twin has to be allocated and filled: not possible while the stream is being captured (the allocation would end
+        // the capture with an error, and a replay would not repeat it).
+        hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+        if (hipError_t e = hipStreamIsCapturing(static_cast<hipStream_t>(stream), &cap); e != hipSuccess) return (int)e;
+        if (cap != hipStreamCaptureStatusNone) return FP6MI_ERR_CAPTURE;
+        size_t bytes = fp6mi::native_bytes(E, Mb, M, K);
+        if (hipError_t e = hipMalloc(&native, bytes); e != hipSuccess) return (int)e;
+        rc = fp6mi_relayout_ref_to_native_gpu(E, Mb, stream, native, W_ref, M, K);
+        // The twin becomes visible to other callers (and other streams) only once it is completely written: this
+        // one-time path waits for the relayout kernel before it publishes the pointer.
+        if (rc == 0) rc = (int)hipStreamSynchronize(static_cast<hipStream_t>(stream));
+        if (rc != 0) {
+            (void)hipFree(native);
+            return rc;
         }
+        void *duplicate = nullptr;
+        {
+            std::lock_guard<std::mutex> lock(g_twin_mutex);
+            auto ins = g_twins.emplace(W_ref, Twin{ native, E, Mb, M, K, device });
+            if (!ins.second) { // another thread converted the same weights meanwhile
+                const Twin &t = ins.first->second;
+                if (t.E == E && t.Mb == Mb && t.M == M && t.K == K && t.device == device) {
+                    duplicate = native;   // keep theirs, which may already be in use
+                    native = t.native;
+                } else {                  // theirs describes another matrix at this address: ours is the newer truth
+                    duplicate = t.native;
+                    ins.first->second = Twin{ native, E, Mb, M, K, device };
+                }
+            }
+        }
+        if (duplicate) (void)hipFree(duplicate);
     }
     return fp6mi_linear_native(E, Mb, stream, native, sc, B, C, M, N, K, ws, splitK);
 }

@@ -676,7 +676,13 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
     // global load sits on the tail of the kernel
     v4h sc4[RT];
 #pragma unroll
-    for (int r = 0; r < RT; r++) sc4[r] = *reinterpret_cast<const v4h *>(scales + (R0 + r) * 16 + 4 * q);
+    for (int r = 0; r < RT; r++) {
+        const half_t *p = scales + (R0 + r) * 16 + 4 * q;
+        if ((reinterpret_cast<uintptr_t>(scales) & 7u) == 0) // uniform: one 8-byte load where the caller's pointer allows it
+            sc4[r] = *reinterpret_cast<const v4h *>(p);
+        else
+            sc4[r] = (v4h){ p[0], p[1], p[2], p[3] };
+    }
 
     tile_segment<FM, GS, NT, RT, WR, WK>(acc, W, gexp, X, N, K, units, mb, nbase, u0, u1, lds, tid, lane, wr, wk, col, q);
 

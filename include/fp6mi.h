@@ -14,7 +14,8 @@
  *   "raw" weights     : row-major [M,K] codes, per-row MSB-first bitstream, M*K*x/8 bytes.
  *   "ref" layout      : the reference's prepacked layout (utils/weight_prepacking.h:118-196), same byte count.
  *   "native" layout   : this engine's gfx950 layout, fp6mi_native_bytes() bytes (K padded to 256).
- *   activations B     : fp16 [N,K] row-major;  output C : fp16 [N,M] row-major;  scales : fp16 [M], 8-byte aligned.
+ *   activations B     : fp16 [N,K] row-major;  output C : fp16 [N,M] row-major;  scales : fp16 [M], 2-byte aligned
+ *   (a view into a larger scale tensor is fine; 8-byte alignment lets the large-batch kernel fetch four at a time).
  *
  * Return value of every int function: 0 on success, a negative FP6MI_ERR_* for rejected arguments, or a positive
  * hipError_t from the runtime.  Nothing here aborts the process.  GPU entry points enqueue on `stream`
@@ -36,7 +37,7 @@ extern "C" {
 #define FP6MI_ERR_NULL (-3)      /* a required pointer is NULL              */
 #define FP6MI_ERR_WORKSPACE (-4) /* splitK > 1 without a workspace          */
 #define FP6MI_ERR_SPLITK (-5)    /* splitK < 1                              */
-#define FP6MI_ERR_ALIGN (-6)     /* a device pointer is not 16-byte aligned (scales: 8-byte) */
+#define FP6MI_ERR_ALIGN (-6)     /* a device pointer is not 16-byte aligned (scales, group exponents: 2-byte) */
 #define FP6MI_ERR_TOO_LARGE (-7) /* the problem exceeds the static workspace of fp6mi_linear_native_static */
 #define FP6MI_ERR_CAPTURE (-8)   /* the call would have to allocate while its stream is being captured */
 
@@ -111,8 +112,10 @@ int    fp6mi_init(void);
  * whose stream is being captured returns FP6MI_ERR_CAPTURE instead of allocating (the reference's entry point
  * allocates nothing, fp6_llm/csrc/fp6_linear.cu:104-117): make the first call, or fp6mi_relayout_ref_to_native_gpu,
  * before the capture.  The twin is keyed by ADDRESS: if the caller overwrites or frees-and-reuses the weight buffer
- * it must call fp6mi_twin_evict(W) (or fp6mi_twin_clear()) first.  Callers that cannot tolerate the hidden
- * allocation convert explicitly and use fp6mi_linear_native. */
+ * it must call fp6mi_twin_evict(W) (or fp6mi_twin_clear()) first.  The first call per weight allocates and synchronizes
+ * `stream` (outside the library's lock: calls on other weights from other threads are not held up), so it must not
+ * overlap another thread's stream capture in global mode.  Callers that cannot tolerate the hidden allocation convert
+ * explicitly and use fp6mi_linear_native. */
 int fp6mi_linear(int E, int Mbits, void *stream, const void *W_ref, const void *scales_f16, const void *B_f16,
                  void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK);
 int fp6mi_twin_evict(const void *W_ref);

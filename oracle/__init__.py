@@ -293,7 +293,9 @@ def dequant_from_definition(codes, scale, E=3, M=2):
 def dequant_grouped_from_definition(codes, scale, exps, E=3, M=2):
     """fp16_rn(value(code) * 2^(b-127) * scale) with one exponent byte b per (row, 128 columns): the definition of this
     build's per-group scales.  The reference has no per-group scales (one half per row, fp6_llm/csrc/fp6_linear.cuh:24), so
-    there is no reference behaviour to pin this against: PARITY UNPINNED, the definition itself is the arbiter."""
+    no reference output exists for it; it is pinned by reduction to the row-scale dequantizer (tests/test_oracle.py): unit
+    exponents give dequant_from_definition, a single exponent b with scale * 2^(b-127) representable gives
+    dequant(raw, scale * 2^(b-127)) bit for bit, and mixed groups give the column blocks of those."""
     tab = value_table(E, M)
     codes = np.asarray(codes)
     f = np.repeat(np.exp2(np.asarray(exps, dtype=np.float64) - 127.0), 128, axis=1)[:, :codes.shape[1]]

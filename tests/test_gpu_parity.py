@@ -485,6 +485,53 @@ def test_graph_capture_replays_match_eager():
             assert torch.equal(out, eager), (N, splitK, rep)
 
 
+def test_reference_named_api_first_use_under_capture_then_eager_before_replay():
+    """linear_forward_cuda on reference-layout weights whose FIRST use is inside a stream capture: the conversion is only
+    recorded there, so nothing may be remembered from it.  An eager call before the first replay must convert for itself and
+    be right; the replay must be right too; and a later eager call still is."""
+    E, M = 3, 2
+    OC, IC, N = 512, 1024, 8
+    raw, sc, x = synth.uniform_problem(840, OC, IC, N, E, M)
+    ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+    packed = fp6.weight_prepacking_cpu(torch.from_numpy(raw)).to(DEV)      # a fresh tensor: never seen by the twin cache
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            y_graph = fp6.linear_forward_cuda(xd, packed, scd, 1)
+    y_eager = fp6.linear_forward_cuda(xd, packed, scd, 1)                  # before any replay
+    torch.cuda.synchronize()
+    check_close(y_eager.cpu().numpy(), ref, "eager call between capture and first replay")
+    g.replay()
+    torch.cuda.synchronize()
+    check_close(y_graph.cpu().numpy(), ref, "first replay")
+    y_later = fp6.linear_forward_cuda(xd, packed, scd, 1)
+    torch.cuda.synchronize()
+    assert torch.equal(y_later, y_eager)
+
+
+@pytest.mark.parametrize("N", [3, 16, 40, 200])
+def test_scales_that_are_a_view_at_an_odd_half_offset(N):
+    """The reference puts no alignment rule on the scales (fp6_linear.cuh:11): rows sliced out of a larger scale tensor
+    start at any multiple of two bytes.  Both kernels must take such a pointer and give the bits of the aligned call."""
+    E, M, OC, IC = 3, 2, 512, 1024
+    raw, sc, x = synth.uniform_problem(850 + N, OC, IC, N, E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    xd = torch.from_numpy(x).to(DEV)
+    big = torch.zeros(OC + 8, dtype=torch.float16, device=DEV)
+    for off in (1, 3):
+        view = big[off:off + OC]
+        view.copy_(torch.from_numpy(sc))
+        assert view.data_ptr() % 8 == 2 * off
+        y = fp6.linear_forward_native(E, M, xd, native, view, OC, 1)
+        y0 = fp6.linear_forward_native(E, M, xd, native, torch.from_numpy(sc).to(DEV), OC, 1)
+        torch.cuda.synchronize()
+        assert torch.equal(y, y0), (N, off)
+    check_close(y.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "offset scales N=%d" % N)
+
+
 def test_module_forward():
     from fp6_llm_amd import module
     w = torch.from_numpy(synth.normal(31, (512, 1024))).float()

@@ -165,7 +165,7 @@ def test_error_codes_instead_of_aborts():
     assert L.fp6mi_linear_native(3, 2, None, p, p, p, p, 256, 1, 64, None, 0) == -5
     assert L.fp6mi_linear_native(3, 2, None, None, p, p, p, 256, 1, 64, None, 1) == -3
     assert L.fp6mi_linear_native(3, 2, None, p + 4, p, p, p, 256, 1, 64, None, 1) == -6  # alignment
-    assert L.fp6mi_linear_native(3, 2, None, p, p + 2, p, p, 256, 1, 64, None, 1) == -6  # scales: 8-byte alignment
+    assert L.fp6mi_linear_native(3, 2, None, p, p + 1, p, p, 256, 1, 64, None, 1) == -6  # scales are halfs: 2-byte alignment
     for code in (-1, -2, -3, -4, -5, -6, -7, -8):
         assert len(L.fp6mi_error_string(code)) > 8
     assert L.fp6mi_workspace_bytes(256, 8, 1) == 0 and L.fp6mi_workspace_bytes(256, 8, 3) == 3 * 256 * 8 * 4

@@ -379,3 +379,72 @@ def test_grouped_quantizer_definition(E, M):
     c_row, s_row = oracle.quantize_from_definition(w, E, M)
     assert (s_row == sc).all() and (codes[:, :128] == c_row[:, :128]).all()
     assert codes[0, 128] == (1 << (x - 1)) - 1      # against scale/4 the value top/4 is the largest code
+
+
+# ------------------------------------------------------------------------------------------------ per-group dequantization
+# The reference scales per row only (fp6_llm/csrc/fp6_linear.cuh:24, utils/weight_dequant.h:30-43), so the grouped dequantizer
+# is pinned by what the mathematics fixes: where the group factor can be folded into a representable row scale it must
+# reproduce the (pinned) row-scale dequantizer bit for bit, and a matrix of mixed groups is the column blocks of those.
+def _foldable_scales(rng, rows, shift):
+    """fp16 scales s such that s * 2^shift is again a normal fp16 number (the product is then exact)."""
+    e = rng.integers(max(-14, -14 - shift) + 1, min(15, 15 - shift) - 1, rows)
+    m = rng.integers(0, 1024, rows)
+    return ((1.0 + m / 1024.0) * np.exp2(e.astype(np.float64))).astype(np.float16)
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_grouped_dequant_with_unit_factors_is_the_row_scale_dequantizer(E, M):
+    rng = np.random.default_rng(7100 + 10 * E + M)
+    codes = rng.integers(0, 1 << (1 + E + M), size=(64, 448), dtype=np.uint8)          # 3.5 groups: the last one is cut
+    sc = rng.uniform(1e-3, 1e-2, 64).astype(np.float16)
+    exps = np.full((64, 4), 127, np.uint8)
+    got = oracle.dequant_grouped_from_definition(codes, sc, exps, E, M).view(np.uint16)
+    assert (got == oracle.dequant_from_definition(codes, sc, E, M).view(np.uint16)).all()
+    assert (got == oracle.dequant(oracle.codes_to_raw(codes, E, M), sc, E, M).view(np.uint16)).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("b", [112, 120, 126, 128, 131])
+def test_grouped_dequant_with_one_factor_folds_into_the_row_scale(E, M, b):
+    """exps == b everywhere and scale * 2^(b-127) representable: the answer is dequant(raw, scale * 2^(b-127)), the C oracle
+    that the exhaustive rational check pins."""
+    rng = np.random.default_rng(7200 + 100 * b + 10 * E + M)
+    codes = np.resize(np.arange(1 << (1 + E + M), dtype=np.uint8), (32, 256))            # every code in every row
+    codes = np.roll(codes, rng.integers(0, 64), axis=1)
+    sc = _foldable_scales(rng, 32, b - 127)
+    folded = (sc.astype(np.float64) * 2.0 ** (b - 127)).astype(np.float16)
+    assert (folded.astype(np.float64) == sc.astype(np.float64) * 2.0 ** (b - 127)).all()  # the fold itself is exact
+    got = oracle.dequant_grouped_from_definition(codes, sc, np.full((32, 2), b, np.uint8), E, M).view(np.uint16)
+    want = oracle.dequant(oracle.codes_to_raw(codes, E, M), folded, E, M).view(np.uint16)
+    assert (got == want).all()
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+def test_grouped_dequant_of_mixed_groups_is_column_blocks_of_folded_ones(E, M):
+    """Each 128-column group with its own exponent equals the same columns of the row-scale dequantizer run with that
+    group's folded scale; a transposed or off-by-one group index, or a wrong sign of the exponent, fails here."""
+    rng = np.random.default_rng(7300 + 10 * E + M)
+    rows, K = 48, 576                                                                     # 4.5 groups
+    codes = rng.integers(0, 1 << (1 + E + M), size=(rows, K), dtype=np.uint8)
+    exps = rng.integers(118, 131, size=(rows, 5)).astype(np.uint8)
+    sc = _foldable_scales(rng, rows, -9)[:]                                                # leaves room for shifts in -9..+3
+    sc = np.where(np.abs(np.log2(sc.astype(np.float64))) < 4, sc, np.float16(0.75))
+    got = oracle.dequant_grouped_from_definition(codes, sc, exps, E, M).view(np.uint16)
+    raw = oracle.codes_to_raw(codes, E, M)
+    for g in range(5):
+        for b in np.unique(exps[:, g]):
+            sel = np.nonzero(exps[:, g] == b)[0]
+            folded = (sc.astype(np.float64) * 2.0 ** (int(b) - 127)).astype(np.float16)
+            assert (folded.astype(np.float64) == sc.astype(np.float64) * 2.0 ** (int(b) - 127)).all()
+            want = oracle.dequant(raw, folded, E, M).view(np.uint16)
+            lo, hi = 128 * g, min(K, 128 * g + 128)
+            assert (got[sel, lo:hi] == want[sel, lo:hi]).all(), (g, int(b))
+
+
+def test_grouped_dequant_hand_values():
+    """e3m2 code 0b001100 is 1.0, 0b011111 is 28: with scale 0.5 and exponents 126 / 129 the values are 0.25, 7 / 2, 56."""
+    codes = np.array([[0b001100] * 128 + [0b011111] * 128], np.uint8)
+    out = oracle.dequant_grouped_from_definition(codes, np.array([0.5], np.float16), np.array([[126, 126]], np.uint8), 3, 2)
+    assert out[0, 0] == np.float16(0.25) and out[0, 128] == np.float16(7.0)
+    out = oracle.dequant_grouped_from_definition(codes, np.array([0.5], np.float16), np.array([[129, 129]], np.uint8), 3, 2)
+    assert out[0, 0] == np.float16(2.0) and out[0, 128] == np.float16(56.0)

@@ -43,6 +43,44 @@ def test_static_workspace_entry_point_matches_the_workspace_one():
     _both(2, 1, 768, 1088, 17, 2, 4103)
 
 
+def test_static_workspace_entry_point_allocates_nothing_and_can_be_captured():
+    """After fp6mi_init the entry point must not touch the allocator: the device's free memory is the same before and after
+    eager calls, and a call with split-K recorded as the only work of a stream capture (where an allocation or a lazy
+    symbol lookup would break the capture) replays to the eager result."""
+    L = _lib.lib()
+    assert L.fp6mi_init() == 0
+    E, M, OC, IC, N, splitK = 3, 2, 1024, 4096, 40, 4
+    raw, sc, x = synth.uniform_problem(4110, OC, IC, N, E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+    eager = torch.empty((N, OC), dtype=torch.float16, device=DEV)
+    got = torch.full((N, OC), float("nan"), dtype=torch.float16, device=DEV)
+
+    def call(stream, out, n=N, k=splitK):
+        return L.fp6mi_linear_native_static(E, M, stream, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), OC, n, IC, k)
+
+    assert call(torch.cuda.current_stream().cuda_stream, eager) == 0       # also loads the kernels' code objects
+    assert call(torch.cuda.current_stream().cuda_stream, eager, 8, 3) == 0
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info()[0]                              # hipMemGetInfo: the driver's view, not torch's pool
+    for _ in range(3):
+        assert call(torch.cuda.current_stream().cuda_stream, eager, 8, 3) == 0
+        assert call(torch.cuda.current_stream().cuda_stream, eager) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info()[0] == free_before
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            assert call(s.cuda_stream, got) == 0
+    for rep in range(2):
+        got.fill_(float("nan"))
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got, eager), rep
+
+
 def test_static_workspace_entry_point_rejects_what_does_not_fit():
     L = _lib.lib()
     p = torch.zeros(64, dtype=torch.float16, device=DEV).data_ptr()
