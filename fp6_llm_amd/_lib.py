@@ -56,6 +56,7 @@ def lib():
         "fp6mi_dequant_grouped": (ci, [ci, ci, vp, vp, sz, sz, vp, vp]),
         "fp6mi_linear_native_grouped": (ci, [ci, ci, vp, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci]),
         "fp6mi_dequant_native_grouped_gpu": (ci, [ci, ci, vp, vp, vp, vp, vp, sz, sz]),
+        "fp6mi_linear_native_grouped_cfg": (ci, [ci, ci, vp, vp, vp, vp, vp, vp, sz, sz, sz, vp, ci, ci, ci, ci, ci, ci]),
         "fp6mi_quantize_native_grouped_gpu": (ci, [ci, ci, vp, vp, vp, vp, vp, ci, sz, sz]),
     }
     for name, (res, args) in sigs.items():
@@ -71,7 +72,7 @@ EXPORTED = ["fp6mi_error_string", "fp6mi_version", "fp6mi_tuning_info", "fp6mi_p
             "fp6mi_heuristic_splitk", "fp6mi_heuristic_splitk_format", "fp6mi_workspace_bytes", "fp6mi_linear_native", "fp6mi_linear_native_cfg", "fp6mi_linear", "fp6mi_linear_stateless", "fp6mi_twin_evict", "fp6mi_twin_clear",
             "fp6mi_linear_native_static", "fp6mi_static_workspace_bytes", "fp6mi_init",
             "fp6mi_relayout_ref_to_native_gpu", "fp6mi_dequant_native_gpu", "fp6mi_quantize_native_gpu", "fp6mi_query_launch", "fp6mi_launch_source",
-            "fp6mi_group_exps_bytes", "fp6mi_pack_group_exps", "fp6mi_dequant_grouped", "fp6mi_linear_native_grouped",
+            "fp6mi_group_exps_bytes", "fp6mi_pack_group_exps", "fp6mi_dequant_grouped", "fp6mi_linear_native_grouped", "fp6mi_linear_native_grouped_cfg",
             "fp6mi_dequant_native_grouped_gpu", "fp6mi_quantize_native_grouped_gpu"]
 
 

@@ -147,7 +147,7 @@ const TuneEntry kTune[] = {
 #include "fp6mi_tuning.inc"
 };
 
-inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (16u * c.rt * (c.kind == 1 ? c.wr : 1u)) == 0; }
+inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (16u * c.rt * (c.kind >= 1 ? c.wr : 1u)) == 0; }
 
 // What the table says about a problem that need not be in it: per splitK the shape expected to be fastest and its expected
 // time.  The batch is rounded UP to a measured batch of the same kernel family (a shape's cost steps at column-tile
@@ -175,7 +175,7 @@ const std::vector<TuneGroup> &tune_groups()
 
 inline double rounds_on_chip(const TuneCfg &c, size_t M, size_t N, int splitK)
 {
-    const size_t TM = (size_t)(c.kind == 1 ? c.wr : 1) * c.rt * 16, TN = (size_t)c.nt * 16;
+    const size_t TM = (size_t)(c.kind >= 1 ? c.wr : 1) * c.rt * 16, TN = (size_t)c.nt * 16;
     const double wgs = (double)(M / TM) * (double)((N + TN - 1) / TN) * splitK;
     // tile kernel: one workgroup per CU, two for four-wavefront workgroups.  Stream kernel: several workgroups share a CU, but
     // they share its memory pipeline too, so what counts is the largest number of workgroups any CU is given.
@@ -301,7 +301,7 @@ int linear_native(const fp6mi::FormatOps &ops, hipStream_t st, const void *W, co
     if (splitK > 1) {
         size_t MN = M * N; // M % 256 == 0, so MN % 4 == 0
         const size_t tile_rows = (size_t)c.wr * c.rt * 16, nblocks = (N + (size_t)c.nt * 16 - 1) / ((size_t)c.nt * 16);
-        const size_t grid = c.kind == 1 && M % tile_rows == 0 ? M / tile_rows * nblocks * splitK : 0;
+        const size_t grid = c.kind >= 1 && M % tile_rows == 0 ? M / tile_rows * nblocks * splitK : 0; // gemm_tile and gemm_ws share the tile order
         if (grid && MN / 4 < ((size_t)1 << 31)) {
             // gemm_tile gave every XCD a run of consecutive triples: reduce where the partial sums lie
             const uint32_t q = (uint32_t)(grid / 8), r = (uint32_t)(grid % 8), per_block = (uint32_t)(nblocks * splitK);
@@ -471,6 +471,18 @@ int fp6mi_linear_native_cfg(int E, int Mb, void *stream, const void *W, const vo
     LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
     hipStream_t st = static_cast<hipStream_t>(stream);
     return linear_native(*fp6mi::ops_for(E, Mb), st, W, sc, nullptr, B, C, M, N, K, ws, splitK, &c);
+}
+
+int fp6mi_linear_native_grouped_cfg(int E, int Mb, void *stream, const void *W, const void *sc, const void *group_exps, const void *B, void *C, size_t M,
+                                    size_t N, size_t K, float *ws, int splitK, int kind, int n_tiles, int row_tiles, int row_waves, int k_waves)
+{
+    int rc = check_gemm_args(E, Mb, W, sc, B, C, M, N, K, ws, splitK);
+    if (rc != FP6MI_OK) return rc;
+    if (!group_exps) return FP6MI_ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(group_exps) & 1u) return FP6MI_ERR_ALIGN;
+    LaunchCfg   c = { kind, n_tiles, row_tiles, row_waves, k_waves };
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return linear_native(*fp6mi::ops_for(E, Mb), st, W, sc, group_exps, B, C, M, N, K, ws, splitK, &c);
 }
 
 int fp6mi_launch_source(int E, int Mb, size_t M, size_t N, size_t K, int splitK)

@@ -604,27 +604,30 @@ __device__ __forceinline__ void tile_segment(v4f (&acc)[RT][NT], const uint8_t *
 typedef _Float16 v4h __attribute__((ext_vector_type(4)));
 template <int NT, int RT, int WR> constexpr size_t tile_stage_bytes(bool partial) { return (size_t)NT * 16 * (WR * RT * 16 * (partial ? 4 : 2) + 16); }
 
-template <int FM, int NT, int RT, int WR, int NTHREADS, typename OutT>
-__device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], OutT *__restrict__ out, uint8_t *stage, bool holds_results,
-                                           uint32_t M, uint32_t N, uint32_t mb, uint32_t nbase, int tid, int wr, int col, int q)
+// first half: a wavefront that holds results scales them and parks them in the stage
+template <int FM, int NT, int RT, int WR, typename OutT>
+__device__ __forceinline__ void tile_park(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], uint8_t *stage, int wr, int col, int q)
+{
+    constexpr int TM = WR * RT * 16, kStride = TM * (int)sizeof(OutT) + 16;
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) {
+            v4f v;
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
+            uint8_t *dst = stage + (16 * t + col) * kStride + ((wr * RT + r) * 16 + 4 * q) * (int)sizeof(OutT);
+            if constexpr (sizeof(OutT) == 2)
+                *reinterpret_cast<v4h *>(dst) = (v4h){ (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
+            else
+                *reinterpret_cast<v4f *>(dst) = v;
+        }
+}
+// second half, after a barrier: every thread of the workgroup stores 16-byte pieces of the stage's columns
+template <int NT, int RT, int WR, int NTHREADS, typename OutT>
+__device__ __forceinline__ void tile_flush(OutT *__restrict__ out, const uint8_t *stage, uint32_t M, uint32_t N, uint32_t mb, uint32_t nbase, int tid)
 {
     constexpr int TM = WR * RT * 16, TN = NT * 16, kStride = TM * (int)sizeof(OutT) + 16, kPer16 = 16 / (int)sizeof(OutT); // outputs per 16 bytes
-    if (holds_results) {
-#pragma unroll
-        for (int r = 0; r < RT; r++)
-#pragma unroll
-            for (int t = 0; t < NT; t++) {
-                v4f v;
-#pragma unroll
-                for (int i = 0; i < 4; i++) v[i] = acc[r][t][i] * ((float)sc4[r][i] * Fmt<FM>::post_scale);
-                uint8_t *dst = stage + (16 * t + col) * kStride + ((wr * RT + r) * 16 + 4 * q) * (int)sizeof(OutT);
-                if constexpr (sizeof(OutT) == 2)
-                    *reinterpret_cast<v4h *>(dst) = (v4h){ (half_t)v[0], (half_t)v[1], (half_t)v[2], (half_t)v[3] };
-                else
-                    *reinterpret_cast<v4f *>(dst) = v;
-            }
-    }
-    __syncthreads();
     constexpr int kPiecesPerCol = TM / kPer16, kPieces = TN * kPiecesPerCol;
 #pragma unroll
     for (int p = tid; p < kPieces; p += NTHREADS) {
@@ -635,6 +638,15 @@ __device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (
             *reinterpret_cast<v4u *>(out + (size_t)ng * M + (size_t)mb * TM + piece * kPer16) = d;
         }
     }
+}
+
+template <int FM, int NT, int RT, int WR, int NTHREADS, typename OutT>
+__device__ __forceinline__ void tile_store(const v4f (&acc)[RT][NT], const v4h (&sc4)[RT], OutT *__restrict__ out, uint8_t *stage, bool holds_results,
+                                           uint32_t M, uint32_t N, uint32_t mb, uint32_t nbase, int tid, int wr, int col, int q)
+{
+    if (holds_results) tile_park<FM, NT, RT, WR, OutT>(acc, sc4, stage, wr, col, q);
+    __syncthreads();
+    tile_flush<NT, RT, WR, NTHREADS, OutT>(out, stage, M, N, mb, nbase, tid);
 }
 
 template <int FM, bool GS, int NT, int RT, int WR, int WK>
@@ -693,6 +705,226 @@ __global__ __launch_bounds__(WR *WK *kWave) void gemm_tile(const uint8_t *__rest
         tile_store<FM, NT, RT, WR, NTHREADS>(acc, sc4, C, stage, wk == 0, M, N, mb, nbase, tid, wr, col, q);
     else
         tile_store<FM, NT, RT, WR, NTHREADS>(acc, sc4, ws + (size_t)split * N * M, stage, wk == 0, M, N, mb, nbase, tid, wr, col, q);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// gemm_ws: the tile GEMM with the wavefronts of a workgroup divided into two kinds.
+//   workgroup = WR arithmetic wavefronts + PW loading wavefronts; tile = (WR*RT*16) rows x (NT*16) columns; same grid as gemm_tile
+// The loading wavefronts move K blocks from memory into LDS without passing through registers (global_load_lds_dwordx4):
+// the tile's weight blocks exactly as they lie in memory (native blocks of raw codes, 16-byte pieces in lane order) and the
+// activation rows of the block.  The arithmetic wavefronts never touch global memory inside the K loop: they read their
+// weight pieces and their B operands from LDS, convert and run the MFMAs.  In gemm_tile every wavefront does both, a
+// wavefront issues its instructions in order, and the CU's memory pipeline accepts a chunk's loads at its own pace: there
+// the second wavefront of every SIMD starts its MFMAs a third of a K step late, and a block has to arrive within the one
+// step before it is used.  Here the weights travel SW-1 blocks ahead of the arithmetic and the activations SX-1 blocks
+// (SW >= SX >= 2: the weights come from HBM, the activations from L2), during the whole of those steps.
+// LDS: a ring of SW weight stages [WR*RT tiles x block bytes] and a ring of SX activation stages [NT*16 rows x 512 bytes].
+// The activation rows are not padded (256 x 64 with FP6 weights and two stages each fills the 160 KB to the byte): piece p
+// of row n (16 bytes) lies at slot p ^ (n & 15) of its row, which makes the operand read of eight batch columns at one K
+// position touch eight different slots.  One barrier per K block: before it the loading wavefronts wait until the NEXT
+// block has landed (s_waitcnt with the number of transfers issued after it: they complete in order).
+// ---------------------------------------------------------------------------------------------------------------
+template <int FM, int NT, int RT, int WR, int SW, int SX> constexpr size_t ws_ring_bytes()
+{
+    return (size_t)SW * WR * RT * Fmt<FM>::block_bytes + (size_t)SX * NT * 16 * 512;
+}
+
+template <int N> __device__ __forceinline__ void wait_transfers_and_barrier()
+{
+    static_assert(N >= 0 && N <= 63, "s_waitcnt vmcnt holds six bits");
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(N) : "memory");
+}
+
+template <int FM, bool GS, int NT, int RT, int WR, int PW, int SW, int SX>
+__global__ __launch_bounds__((WR + PW) * kWave) void gemm_ws(const uint8_t *__restrict__ W, const half_t *__restrict__ scales,
+                                                             const uint8_t *__restrict__ gexp, const half_t *__restrict__ X, half_t *__restrict__ C,
+                                                             float *__restrict__ ws, uint32_t M, uint32_t N, uint32_t K,
+                                                             uint32_t units, uint32_t splitK, uint32_t nblocks)
+{
+    static_assert(SW >= SX && SX >= 2, "weights run at least as far ahead as activations; a stage is filled while another is read");
+    constexpr int TN = NT * 16, TILES = WR * RT, NTHREADS = (WR + PW) * kWave;
+    constexpr int kBlock = Fmt<FM>::block_bytes, kWStage = TILES * kBlock, kXStage = TN * 512, kXRing = SW * kWStage; // the activation ring follows the weight ring
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+
+    asm volatile("" ::"s"(W), "s"(scales), "s"(gexp), "s"(X), "s"(C), "s"(ws), "s"(M), "s"(N), "s"(K), "s"(units), "s"(splitK), "s"(nblocks)); // one batch of argument loads
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int col = lane & 15, q = lane >> 4;
+
+    // grid.x -> (row block, split, column block), every XCD a run of consecutive triples: as in gemm_tile
+    uint32_t id = blockIdx.x;
+    {
+        const uint32_t per = gridDim.x >> 3, r = gridDim.x & 7u, x = id & 7u;
+        id = x * per + (x < r ? x : r) + (id >> 3);
+    }
+    const uint32_t nb = id % nblocks, rest = id / nblocks, split = rest % splitK, mb = rest / splitK;
+    const uint32_t nbase = nb * TN;
+    uint32_t       u0 = 0, u1 = units;
+    if (splitK > 1) {
+        const uint32_t avg = units / splitK, extra = units % splitK;
+        u0 = split * avg + (split < extra ? split : extra);
+        u1 = u0 + avg + (split < extra ? 1u : 0u);
+    }
+    const int nk = (int)(u1 - u0); // K blocks of this workgroup, numbered 0 .. nk-1 below
+
+    v4f acc[RT][NT];
+    v4h sc4[RT];
+#pragma unroll
+    for (int r = 0; r < RT; r++)
+#pragma unroll
+        for (int t = 0; t < NT; t++) acc[r][t] = (v4f){ 0.f, 0.f, 0.f, 0.f };
+
+    if (wave >= WR) {
+        // ---------------------------------------------------------------- loading wavefronts
+        // One instruction moves 64 x 16 bytes from memory straight into 1 KB of LDS, lane l to byte 16*l of the destination;
+        // each lane chooses its source address.  Instruction i of a weight (activation) stage fills its pieces 64*i .. 64*i+63;
+        // this wavefront issues the instructions pw, pw + PW, ...
+        typedef __attribute__((address_space(1))) void gvoid;
+        typedef __attribute__((address_space(3))) void lvoid;
+        const int     pw = wave - WR;
+        constexpr int PB = kBlock / 16, kWPieces = TILES * PB, kXPieces = TN * 32;
+        static_assert(kWPieces % 64 == 0 && kXPieces % 64 == 0, "a stage is a whole number of 1 KB instructions");
+        constexpr int kWInst = kWPieces / 64, kXInst = kXPieces / 64;
+        static_assert(kWInst % PW == 0 && kXInst % PW == 0, "every loading wavefront issues the same number of transfers (the waits count them)");
+        constexpr int kWPer = kWInst / PW, kXPer = kXInst / PW;
+        // transfers issued after those of block j+1 when step j ends: the later of its two transfers is the activation one, issued
+        // SX-2 steps ago and followed there by that step's weight transfers when the weight ring is the deeper one
+        constexpr int kAhead = (SW > SX ? kWPer : 0) + (SX - 2) * (kWPer + kXPer);
+        // weight piece P (16 bytes) of a stage = piece P % PB of the block of tile P / PB: a straight copy
+        const uint8_t *wsrc[kWPer];
+#pragma unroll
+        for (int j = 0; j < kWPer; j++) {
+            const uint32_t P = (pw + PW * j) * 64 + lane, tile = P / PB, within = P % PB;
+            wsrc[j] = W + ((size_t)(mb * TILES + tile) * units + u0) * kBlock + within * 16;
+        }
+        // activation piece P of a stage = slot P % 32 of row P / 32, which holds piece slot ^ (row & 15) of that batch column's
+        // 256 halfs (columns beyond N repeat the last real one: their outputs are never stored)
+        const uint8_t *xsrc[kXPer];
+        uint32_t       xpiece[kXPer];
+#pragma unroll
+        for (int j = 0; j < kXPer; j++) {
+            const uint32_t P = (pw + PW * j) * 64 + lane, n = P >> 5, piece = (P & 31) ^ (n & 15);
+            const uint32_t row = nbase + n < N ? nbase + n : N - 1;
+            xsrc[j] = reinterpret_cast<const uint8_t *>(X + (size_t)row * K + (size_t)u0 * 256) + piece * 16;
+            xpiece[j] = piece;
+        }
+        auto fetch_w = [&](int k, int slot) { // weights of block k -> stage `slot` of the weight ring
+            uint8_t *st = lds + slot * kWStage;
+#pragma unroll
+            for (int j = 0; j < kWPer; j++)
+                __builtin_amdgcn_global_load_lds((gvoid *)(wsrc[j] + (size_t)k * kBlock), (lvoid *)(st + (pw + PW * j) * 1024), 16, 0, 0);
+        };
+        auto fetch_x = [&](int k, int slot) { // activations of block k -> stage `slot` of the activation ring
+            uint8_t *st = lds + kXRing + slot * kXStage;
+            if ((u0 + k + 1) * 256 <= K) {
+#pragma unroll
+                for (int j = 0; j < kXPer; j++)
+                    __builtin_amdgcn_global_load_lds((gvoid *)(xsrc[j] + (size_t)k * 512), (lvoid *)(st + (pw + PW * j) * 1024), 16, 0, 0);
+            } else { // the block that K cuts goes through registers: positions beyond K are read at the block's start (a valid address) and stored as zeros
+#pragma unroll
+                for (int j = 0; j < kXPer; j++) {
+                    const bool ok = (u0 + k) * 256 + xpiece[j] * 8 < K;
+                    const v4u  v = *reinterpret_cast<const v4u *>(xsrc[j] + (size_t)k * 512 - (ok ? 0u : xpiece[j] * 16));
+                    *reinterpret_cast<v4u *>(st + (pw + PW * j) * 1024 + lane * 16) = ok ? v : (v4u){ 0u, 0u, 0u, 0u };
+                }
+            }
+        };
+        if (nk > 0) {
+            // step j (j = -(SW-1) .. nk-1; the negative ones fill the rings) issues the activations of block j+SX-1 and then the
+            // weights of block j+SW-1; it ends with a barrier before which block j+1 must have landed
+            int wslot = 0, xslot = 0; // ring positions the next transfers go to
+            for (int j = 1 - SW; j < nk; j++) {
+                const int kx = j + SX - 1, kw = j + SW - 1;
+                if (kx >= 0 && kx < nk) {
+                    fetch_x(kx, xslot);
+                    xslot = xslot + 1 == SX ? 0 : xslot + 1;
+                }
+                if (kw < nk) {
+                    fetch_w(kw, wslot);
+                    wslot = wslot + 1 == SW ? 0 : wslot + 1;
+                }
+                if (j >= -1) {
+                    // the count is exact only while every transfer it assumes was issued; at the end of K wait for everything
+                    // (block j+1's last transfer is followed by exactly kAhead others as long as this step still had weights to fetch)
+                    if (kw < nk)
+                        wait_transfers_and_barrier<kAhead>();
+                    else
+                        wait_transfers_and_barrier<0>();
+                }
+            }
+        }
+    } else {
+        // ---------------------------------------------------------------- arithmetic wavefronts
+        const int      wr = wave;
+        const uint32_t R0 = (mb * WR + wr) * RT; // first row tile of this wavefront
+#pragma unroll
+        for (int r = 0; r < RT; r++) {
+            const half_t *p = scales + (R0 + r) * 16 + 4 * q;
+            if ((reinterpret_cast<uintptr_t>(scales) & 7u) == 0)
+                sc4[r] = *reinterpret_cast<const v4h *>(p);
+            else
+                sc4[r] = (v4h){ p[0], p[1], p[2], p[3] };
+        }
+        const uint8_t *ggroup = GS ? gexp + ((size_t)R0 * units + u0) * 32 : nullptr;
+        uint32_t       xoff[8]; // B operand of MFMA step s: row col, piece 4s+q, at its swizzled slot
+#pragma unroll
+        for (int s8 = 0; s8 < 8; s8++) xoff[s8] = kXRing + col * 512 + 16 * ((4 * s8 + q) ^ col);
+        const uint32_t woff = wr * RT * kBlock + lane * 16;
+        if (nk > 0) {
+            uint32_t gnext[RT];
+#pragma unroll
+            for (int r = 0; r < RT; r++) gnext[r] = load_group_exps<GS>(ggroup, (size_t)r * units, lane);
+            __syncthreads(); // block 0 has landed
+            int wslot = 0, xslot = 0;
+            for (int k = 0; k < nk; k++) {
+                const uint8_t *wst = lds + wslot * kWStage, *xst = lds + xslot * kXStage;
+                wslot = wslot + 1 == SW ? 0 : wslot + 1;
+                xslot = xslot + 1 == SX ? 0 : xslot + 1;
+                WFrag<FM> wf[RT];
+                uint32_t  g[RT];
+#pragma unroll
+                for (int r = 0; r < RT; r++) {
+                    const uint8_t *b = wst + woff + r * kBlock;
+                    wf[r].a = *reinterpret_cast<const v4u *>(b);
+                    wf[r].b = *reinterpret_cast<const v4u *>(b + 1024);
+                    if constexpr (Fmt<FM>::bits == 6) wf[r].c = *reinterpret_cast<const v4u *>(b + 2048);
+                    if constexpr (Fmt<FM>::bits == 5) wf[r].s = *reinterpret_cast<const v2u *>(wst + (wr * RT + r) * kBlock + 2048 + lane * 8);
+                    g[r] = gnext[r];
+                    if (GS && k + 1 < nk) gnext[r] = load_group_exps<GS>(ggroup, (size_t)r * units + k + 1, lane);
+                }
+                v8h a0[RT][4], a1[RT][4];
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wf[r], 0, a0[r], g[r]);
+#pragma unroll
+                for (int r = 0; r < RT; r++) convert_half<FM, GS>(wf[r], 1, a1[r], g[r]);
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+#pragma unroll
+                    for (int s = 0; s < 4; s++) {
+                        v8h b[NT];
+#pragma unroll
+                        for (int t = 0; t < NT; t++) b[t] = *reinterpret_cast<const v8h *>(xst + xoff[4 * h + s] + t * 16 * 512);
+#pragma unroll
+                        for (int r = 0; r < RT; r++)
+#pragma unroll
+                            for (int t = 0; t < NT; t++)
+                                acc[r][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(h == 0 ? a0[r][s] : a1[r][s], b[t], acc[r][t], 0, 0, 0);
+                    }
+                }
+                __syncthreads();
+            }
+        }
+    }
+    // every wavefront has passed the last barrier of the K loop: the rings are free, the output tile is parked there
+    uint8_t *stage = lds;
+    if (splitK == 1) {
+        if (wave < WR) tile_park<FM, NT, RT, WR, half_t>(acc, sc4, stage, wave, col, q);
+        __syncthreads();
+        tile_flush<NT, RT, WR, NTHREADS, half_t>(C, stage, M, N, mb, nbase, tid);
+    } else {
+        if (wave < WR) tile_park<FM, NT, RT, WR, float>(acc, sc4, stage, wave, col, q);
+        __syncthreads();
+        tile_flush<NT, RT, WR, NTHREADS, float>(ws + (size_t)split * N * M, stage, M, N, mb, nbase, tid);
+    }
 }
 
 // Native layout -> fp16 [M,K], with the GEMM's own conversion code.  One lane per (row tile, K block, lane) triple.
@@ -1010,7 +1242,34 @@ int launch_tile(hipStream_t st, const void *W, const void *sc, const void *gexp,
                        static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
     return (int)hipGetLastError();
 }
-// kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts)
+template <int FM, bool GS, int NT, int RT, int WR, int PW, int SW, int SX>
+int launch_ws(hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M, size_t N, size_t K,
+              int splitK)
+{
+    constexpr int    TN = NT * 16, TM = WR * RT * 16;
+    constexpr size_t kLoopLds = ws_ring_bytes<FM, NT, RT, WR, SW, SX>(), out_max = tile_stage_bytes<NT, RT, WR>(true);
+    constexpr size_t kMaxLds = kLoopLds > out_max ? kLoopLds : out_max;
+    static_assert(kMaxLds <= 160 * 1024, "the rings do not fit in LDS");
+    static_assert((WR + PW) * kWave <= 1024, "too many wavefronts");
+    // a weight stage must be a whole number of 1 KB transfers per loading wavefront (FP5 blocks are 2.5 KB: 64-row tiles are out)
+    constexpr bool kDivides = (WR * RT * Fmt<FM>::block_bytes) % (1024 * PW) == 0 && (TN * 512) % (1024 * PW) == 0;
+    if constexpr (!kDivides) {
+        return FP6MI_ERR_SHAPE;
+    } else {
+        const size_t out_bytes = tile_stage_bytes<NT, RT, WR>(splitK > 1), lds_bytes = kLoopLds > out_bytes ? kLoopLds : out_bytes;
+        if (M % TM) return FP6MI_ERR_SHAPE;
+        if (kMaxLds > 48 * 1024)
+            if (int rc = allow_dynamic_lds<&gemm_ws<FM, GS, NT, RT, WR, PW, SW, SX>>(kMaxLds)) return rc;
+        uint32_t units = (uint32_t)((K + 255) / 256), nblocks = (uint32_t)((N + TN - 1) / TN);
+        size_t   wgs = (M / TM) * (size_t)splitK * nblocks;
+        if (wgs > 0x7fffffffu) return FP6MI_ERR_SHAPE;
+        hipLaunchKernelGGL((gemm_ws<FM, GS, NT, RT, WR, PW, SW, SX>), dim3((uint32_t)wgs), dim3((WR + PW) * kWave), lds_bytes, st,
+                           static_cast<const uint8_t *>(W), static_cast<const half_t *>(sc), static_cast<const uint8_t *>(gexp), static_cast<const half_t *>(B),
+                           static_cast<half_t *>(C), ws, (uint32_t)M, (uint32_t)N, (uint32_t)K, units, (uint32_t)splitK, nblocks);
+        return (int)hipGetLastError();
+    }
+}
+// kind 0: gemm_stream (wr == 1, wk = wavefronts per workgroup);  kind 1: gemm_tile (wr x wk wavefronts);  kind 2: gemm_ws (wr arithmetic + wk loading wavefronts)
 template <int FM, bool GS>
 int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc, const void *gexp, const void *B, void *C, float *ws, size_t M,
                size_t N, size_t K, int splitK)
@@ -1030,6 +1289,13 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
         FP6MI_CASE(2, 1, 4, 4) FP6MI_CASE(2, 2, 4, 4) FP6MI_CASE(2, 2, 4, 2) FP6MI_CASE(2, 2, 4, 1) FP6MI_CASE(2, 4, 4, 1) FP6MI_CASE(2, 4, 4, 2)
         FP6MI_CASE(4, 2, 4, 2) FP6MI_CASE(4, 2, 4, 1) FP6MI_CASE(4, 4, 4, 1) FP6MI_CASE(4, 4, 2, 1) FP6MI_CASE(4, 4, 2, 2)
         FP6MI_CASE(8, 2, 4, 1) FP6MI_CASE(8, 2, 2, 1) FP6MI_CASE(4, 2, 8, 1) FP6MI_CASE(4, 2, 8, 2) FP6MI_CASE(2, 2, 8, 1) FP6MI_CASE(2, 2, 8, 2) FP6MI_CASE(8, 2, 8, 1) FP6MI_CASE(4, 1, 8, 2) FP6MI_CASE(4, 1, 8, 1) FP6MI_CASE(4, 1, 4, 2) FP6MI_CASE(2, 1, 2, 4)
+#undef FP6MI_CASE
+    } else if (c.kind == 2) {
+        // ring depths (2,2): deeper rings on smaller tiles (128 x 64 with (4,2), 128 x 32 and 64 x 64 with (4,3)) measured no faster than
+        // gemm_tile at batches 32-64, where the time goes to the partial sums and the second launch, and are not built
+#define FP6MI_CASE(NT, RT, WR, PW) \
+    if (c.nt == NT && c.rt == RT && c.wr == WR && c.wk == PW) return launch_ws<FM, GS, NT, RT, WR, PW, 2, 2>(st, W, sc, gexp, B, C, ws, M, N, K, splitK);
+        FP6MI_CASE(4, 2, 8, 4) FP6MI_CASE(4, 2, 4, 4) FP6MI_CASE(2, 2, 8, 4)
 #undef FP6MI_CASE
     }
     return FP6MI_ERR_SHAPE;

@@ -24,7 +24,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 INC_PATH = os.path.join(HERE, "csrc", "fp6mi_tuning.inc")
 
-# (kind, n_tiles, row_tiles, row_waves, k_waves); kind 0 = stream kernel (batch <= 16 per n_tile), 1 = tile kernel
+# (kind, n_tiles, row_tiles, row_waves, k_waves); kind 0 = stream kernel (batch <= 16 per n_tile), 1 = tile kernel, 2 = wave-specialized tile kernel
 STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 4) for wk in (4, 8, 16) if (rt, wk) != (4, 16)]
 STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4)]                      # two 16-column tiles per workgroup, batches 17..32
 TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
@@ -41,6 +41,19 @@ COMPILED_TILE = [(1,) + c for c in
                  [(2, 1, 4, 4), (2, 2, 4, 4), (2, 2, 4, 2), (2, 2, 4, 1), (2, 4, 4, 1), (2, 4, 4, 2), (4, 2, 4, 2), (4, 2, 4, 1), (4, 4, 4, 1),
                   (4, 4, 2, 1), (4, 4, 2, 2), (8, 2, 4, 1), (8, 2, 2, 1), (4, 2, 8, 1), (4, 2, 8, 2), (2, 2, 8, 1), (2, 2, 8, 2), (8, 2, 8, 1),
                   (4, 1, 8, 2), (4, 1, 8, 1), (4, 1, 4, 2), (2, 1, 2, 4)]]
+
+# kind 2 = wave-specialized tile kernel: (2, n_tiles, row_tiles, arithmetic wavefronts, loading wavefronts)
+COMPILED_WS = [(2, 4, 2, 8, 4), (2, 4, 2, 4, 4), (2, 2, 2, 8, 4)]
+
+BLOCK_BYTES = {6: 3072, 5: 2560, 4: 2048}   # one native 16-row x 256-column block per bit width
+
+
+def shape_compiled_for(cfg, bits):
+    """Every stream and tile shape exists for every format; a wave-specialized shape needs its weight stage to be a whole number
+    of 1 KB transfers per loading wavefront (FP5 blocks are 2.5 KB, so its 64-row tiles are out)."""
+    kind, nt, rt, wr, wk = cfg
+    return kind < 2 or (wr * rt * BLOCK_BYTES[bits]) % (1024 * wk) == 0
+
 
 GRID_M = [1024, 2048, 3072, 4096, 5120, 6144, 8192, 10240, 11008, 12288, 14336, 16384, 22016, 28672, 32768]
 GRID_K = [2048, 4096, 5120, 8192, 11008, 14336, 28672]
@@ -65,26 +78,31 @@ MODEL_PAIRS = [(15360, 5120), (13824, 5120), (27648, 5120), (5120, 13824), (7168
 
 def tile_rows(cfg):
     kind, nt, rt, wr, wk = cfg
-    return 16 * rt * (wr if kind == 1 else 1)
+    return 16 * rt * (wr if kind >= 1 else 1)
 
 
-def candidates(OC, IC, BS, kinds=None, splits=None):
-    """(shape, splitK) pairs worth measuring; `kinds` ("stream", "tile") and `splits` narrow the list for a partial sweep."""
-    for cfg, sk in _all_candidates(OC, IC, BS):
-        if kinds and ("stream" if cfg[0] == 0 else "tile") not in kinds:
+KIND_NAMES = ("stream", "tile", "ws")
+
+
+def candidates(OC, IC, BS, kinds=None, splits=None, bits=6):
+    """(shape, splitK) pairs worth measuring; `kinds` ("stream", "tile", "ws") and `splits` narrow the list for a partial sweep."""
+    for cfg, sk in _all_candidates(OC, IC, BS, bits):
+        if kinds and KIND_NAMES[cfg[0]] not in kinds:
             continue
         if splits and sk not in splits:
             continue
         yield cfg, sk
 
 
-def _all_candidates(OC, IC, BS):
+def _all_candidates(OC, IC, BS, bits=6):
     if BS <= 16:
         cfgs = STREAM_SMALL
     else:
         cfgs = [c for c in TILE if (c[1] * 16 < 2 * BS + 16 or c[1] == 2) and (BS <= 512 or c[1] >= 4)]
         if BS <= 32:
             cfgs = cfgs + STREAM_WIDE
+        if BS >= 96:    # the wave-specialized tiles pay from about 128 columns up (256 x 64 from 256 up on 8192 x 8192)
+            cfgs = cfgs + [c for c in COMPILED_WS if c[1] * 16 <= BS]
     units = (IC + 255) // 256
     for cfg in cfgs:
         if OC % tile_rows(cfg):
@@ -179,13 +197,13 @@ def sweep(args):
                     continue
                 for BS in Ns:
                     best = {}
-                    for cfg, sk in candidates(OC, IC, BS, kinds, splits):
+                    for cfg, sk in candidates(OC, IC, BS, kinds, splits, args.format):
                         t = bench(E, M, OC, IC, BS, cfg, sk)
                         if t is not None and (str(sk) not in best or t < best[str(sk)][1]):
                             best[str(sk)] = [list(cfg), round(t, 3)]
                     row = {"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best, "lib": bench.lib_version, "rocm": bench.rocm}
                     if kinds or splits:   # a partial row: `merge` folds it into a full one
-                        row["partial"] = {"kinds": sorted(kinds) if kinds else ["stream", "tile"], "splits": sorted(splits) if splits else list(SPLITS)}
+                        row["partial"] = {"kinds": sorted(kinds) if kinds else list(KIND_NAMES), "splits": sorted(splits) if splits else list(SPLITS)}
                     f.write(json.dumps(row) + "\n")
                     f.flush()
                     print("e%dm%d %dx%d N=%d: " % (E, M, OC, IC, BS) + "  ".join("sk%s %s %.2f" % (k, "".join(map(str, v[0])), v[1]) for k, v in best.items()),
@@ -235,12 +253,12 @@ def merge(args):
         for line in open(path):
             p = json.loads(line)
             key = (p["E"], p["M"], p["OC"], p["IC"], p["BS"])
-            part = p.get("partial", {"kinds": ["stream", "tile"], "splits": list(SPLITS)})
+            part = p.get("partial", {"kinds": list(KIND_NAMES), "splits": list(SPLITS)})
             old = rows.get(key, {"E": p["E"], "M": p["M"], "OC": p["OC"], "IC": p["IC"], "BS": p["BS"], "best": {}})
             best = {}
             for sk in sorted(set(old["best"]) | set(p["best"]), key=int):
                 o, n = old["best"].get(sk), p["best"].get(sk)
-                if o is not None and int(sk) in part["splits"] and ("stream" if o[0][0] == 0 else "tile") in part["kinds"]:
+                if o is not None and int(sk) in part["splits"] and KIND_NAMES[o[0][0]] in part["kinds"]:
                     o = None   # re-measured: whatever the old entry says about this kind is out of date
                 cands = [c for c in (o, n) if c is not None]
                 if cands:
@@ -282,7 +300,7 @@ def main(argv=None):
     s.add_argument("--k", default="")
     s.add_argument("--n", default="")
     s.add_argument("--pairs", default="", help="OCxIC,OCxIC,... instead of the m x k grid, or `models` for the built-in list of layer shapes")
-    s.add_argument("--kinds", default="", help="stream, tile or both (comma-separated): measure only these kernels' shapes (the rows are partial: see merge)")
+    s.add_argument("--kinds", default="", help="stream, tile, ws (comma-separated): measure only these kernels' shapes (the rows are partial: see merge)")
     s.add_argument("--splits", default="", help="measure only these splitK values (the rows are partial: see merge)")
     s.add_argument("--iters", type=int, default=30)
     s.add_argument("--reps", type=int, default=5)

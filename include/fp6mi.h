@@ -133,12 +133,19 @@ int fp6mi_linear_stateless(int E, int Mbits, void *stream, const void *W_ref, co
 /* Tuning hook: the same GEMM with the launch shape chosen by the caller instead of the built-in selection
  * (no counterpart in the reference, whose TilingConfig is picked inside fpx_linear_kernel, fp6_linear.cu:61-81).
  * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup),
- * kind 1 = tile kernel (row_waves x k_waves wavefronts, activations staged in LDS);
+ * kind 1 = tile kernel (row_waves x k_waves wavefronts, activations staged in LDS),
+ * kind 2 = wave-specialized tile kernel (row_waves arithmetic wavefronts; k_waves = 4 loading wavefronts that move weights and
+ *          activations into LDS for them);
  * n_tiles = 16-column batch tiles per workgroup, row_tiles = 16-row weight tiles per wavefront.
  * Combinations that are not compiled in, or that do not divide M, return FP6MI_ERR_SHAPE. */
 int fp6mi_linear_native_cfg(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
                             const void *B_f16, void *C_f16, size_t M, size_t N, size_t K, float *workspace, int splitK,
                             int kind, int n_tiles, int row_tiles, int row_waves, int k_waves);
+
+/* The same hook for weights with group exponents (fp6mi_linear_native_grouped with the launch shape chosen by the caller). */
+int fp6mi_linear_native_grouped_cfg(int E, int Mbits, void *stream, const void *W_native, const void *scales_f16,
+                                    const void *group_exps_native, const void *B_f16, void *C_f16, size_t M, size_t N, size_t K,
+                                    float *workspace, int splitK, int kind, int n_tiles, int row_tiles, int row_waves, int k_waves);
 
 /* Which kernel shape fp6mi_linear_native would launch for this problem: shape[0..4] = kind, n_tiles, row_tiles,
  * row_waves, k_waves, with the meaning they have in fp6mi_linear_native_cfg.  Pure host code, no GPU needed.  The

@@ -130,20 +130,59 @@ def test_split_k(E, M, splitK):
     check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "splitK=%d" % splitK)
 
 
-from fp6_llm_amd.tune import COMPILED_STREAM as STREAM_SHAPES, COMPILED_TILE as TILE_SHAPES  # noqa: E402
+from fp6_llm_amd.tune import COMPILED_STREAM as STREAM_SHAPES, COMPILED_TILE as TILE_SHAPES, COMPILED_WS as WS_SHAPES, shape_compiled_for as tune_shape_compiled_for, tile_rows as tune_tile_rows  # noqa: E402
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
-@pytest.mark.parametrize("cfg", STREAM_SHAPES + TILE_SHAPES)
+@pytest.mark.parametrize("cfg", STREAM_SHAPES + TILE_SHAPES + WS_SHAPES)
 def test_every_launch_shape(E, M, cfg):
     """Every compiled (kernel, tile) combination through the tuning hook: cfg = (kind, n_tiles, row_tiles, row_waves, k_waves)."""
     print("case launch shape", E, M, cfg, flush=True)
+    if not tune_shape_compiled_for(cfg, 1 + E + M):
+        pytest.skip("this shape is not built for this bit width")
     OC, IC, N = 512, 2304, 16 * cfg[1] - 3
     raw, sc, x = synth.uniform_problem(500 + sum(cfg), OC, IC, N, E, M)
     native, scd, xd = upload(raw, sc, x, E, M)
     ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
     for splitK in (1, 3):
         check_close(gemm_capi(E, M, native, scd, xd, OC, splitK, cfg), ref, "cfg %s splitK %d" % (cfg, splitK))
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("cfg", WS_SHAPES)
+def test_wave_specialized_kernel_edges(E, M, cfg):
+    """The kernel whose loading wavefronts fill LDS rings for its arithmetic wavefronts, where its bookkeeping is thinnest: a K
+    that ends inside a block (that block's activations take the register path), batch columns that end inside a column tile,
+    splits with fewer K blocks than the rings are deep (one block, and none at all), and weights with group exponents."""
+    print("case wave-specialized edges", E, M, cfg, flush=True)
+    if not tune_shape_compiled_for(cfg, 1 + E + M):
+        pytest.skip("this shape is not built for this bit width")
+    L = _lib.lib()
+    OC = 2 * tune_tile_rows(cfg)
+    for (IC, N, splits) in [(1088, 16 * cfg[1] + 6, (1, 2, 5)), (320, 3, (1, 3)), (4160, 16 * cfg[1] - 1, (1, 4))]:
+        raw, sc, x = synth.uniform_problem(600 + IC + sum(cfg), OC, IC, N, E, M)
+        native, scd, xd = upload(raw, sc, x, E, M)
+        ref = oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x)
+        for splitK in splits:
+            y = gemm_capi(E, M, native, scd, xd, OC, splitK, cfg)
+            assert np.isfinite(y).all()
+            check_close(y, ref, "cfg %s IC %d N %d splitK %d" % (cfg, IC, N, splitK))
+    IC, N = 1344, 40
+    codes, sc, ex = quant.quantize_groupwise(_grouped_weights(OC + IC, OC, IC), E, M)
+    wdq = oracle.dequant_grouped_from_definition(codes, sc, ex, E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(quant.pack_raw(codes, E, M))).to(DEV)
+    gexp = fp6.pack_group_exps(torch.from_numpy(ex), OC, IC).to(DEV)
+    scd = torch.from_numpy(sc).to(DEV)
+    x = synth.activations(9, N, IC)
+    xd = torch.from_numpy(x).to(DEV)
+    for splitK in (1, 2):
+        out = torch.full((N, OC), float("nan"), dtype=torch.float16, device=DEV)
+        ws = torch.empty(splitK * N * OC, dtype=torch.float32, device=DEV)
+        rc = L.fp6mi_linear_native_grouped_cfg(E, M, torch.cuda.current_stream().cuda_stream, native.data_ptr(), scd.data_ptr(), gexp.data_ptr(),
+                                               xd.data_ptr(), out.data_ptr(), OC, N, IC, ws.data_ptr(), splitK, *cfg)
+        assert rc == 0, L.fp6mi_error_string(rc)
+        torch.cuda.synchronize()
+        check_close(out.cpu().numpy(), oracle.gemm_f64(wdq, x), "grouped, cfg %s splitK %d" % (cfg, splitK))
 
 
 @pytest.mark.parametrize("OC,cfg,N,splitK", [

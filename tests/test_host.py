@@ -221,14 +221,16 @@ def test_compiled_launch_shape_lists_match_the_kernel_source():
     from fp6_llm_amd import tune
     src = open(os.path.join(os.path.dirname(fp6.__file__), "csrc", "fp6mi_gemm.hip")).read()
     stream = {(0, int(a), int(b), 1, int(c)) for a, b, c in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+)\)", src)}
-    tile = {(1, int(a), int(b), int(c), int(d)) for a, b, c, d in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+), (\d+)\)", src)}
-    assert stream == set(tune.COMPILED_STREAM) and tile == set(tune.COMPILED_TILE)
+    tile_src, ws_src = src.split("c.kind == 2")    # the wave-specialized shapes are listed after those of the tile kernel
+    tile = {(1, int(a), int(b), int(c), int(d)) for a, b, c, d in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+), (\d+)\)", tile_src)}
+    ws = {(2, int(a), int(b), int(c), int(d)) for a, b, c, d in re.findall(r"FP6MI_CASE\((\d+), (\d+), (\d+), (\d+)\)", ws_src)}
+    assert stream == set(tune.COMPILED_STREAM) and tile == set(tune.COMPILED_TILE) and ws == set(tune.COMPILED_WS)
     assert set(tune.STREAM_SMALL + tune.STREAM_WIDE) <= stream and set(tune.TILE) <= tile
 
 
 def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it():
     from fp6_llm_amd import tune
-    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE)
+    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE + tune.COMPILED_WS)
     inc = open(tune.INC_PATH).read()
     entries = re.findall(r"^\{(\d+),(\d+),(\d+),(\d+),\{(.*)\}\},$", inc, flags=re.M)
     L = _lib.lib()
@@ -485,7 +487,7 @@ def test_bench_refuses_more_than_one_gpu_and_lists_the_benchmark_configurations(
 
 def test_tuner_candidates_and_table_emission(tmp_path, monkeypatch):
     from fp6_llm_amd import tune
-    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE)
+    compiled = set(tune.COMPILED_STREAM + tune.COMPILED_TILE + tune.COMPILED_WS)
     for (OC, IC, BS) in [(256, 64, 1), (4096, 4096, 8), (4096, 4096, 17), (11008, 4096, 64), (768, 2048, 512), (8192, 8192, 2048)]:
         cands = list(tune.candidates(OC, IC, BS))
         assert cands, (OC, IC, BS)
