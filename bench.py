@@ -12,7 +12,8 @@ untimed for ~60 ms (right after an idle spell the GPU runs 10-15 % slow); then t
 many times as it takes to cover ~10 ms, between ONE pair of events, five times over, and the median is reported as time per
 step = event time / (replays x steps in the graph); a graph holds the K steps several times over when K is small -- a
 20-step graph would spread the 6-8 us between two replays over only 20 kernels of 5 us.  The FP16 baseline and the read-only floor are timed the same way.
-The default run also times one workload per benchmark configuration (`detail.configs`) beside an FP16 GEMM of its shape.
+The default run also times every point of the benchmark configurations (`detail.configs`, 29 workloads) beside an FP16 GEMM of
+its shape, and one large FP16 library GEMM as the measured MFMA rate of this GPU (`detail.fp16_peak_tflops_measured`).
 
 Prints ONE JSON line: value = weight bytes streamed per second (the bandwidth figure the reference's design is judged
 on), ms_per_step = time per GEMM; `roofline` prices the GEMM kernel against the 8 TB/s HBM peak from HIP-event time on the
@@ -77,16 +78,16 @@ def algorithmic_bytes(E, M, OC, IC, BS):
     return weight_bytes(E, M, OC, IC) + 2 * OC + 2 * BS * IC + 2 * BS * OC
 
 
-class Problem:
-    """Device buffers of one workload: a pool of native-layout weight buffers, scales, activations, output, workspace."""
+class WeightPool:
+    """Native-layout weight buffers of one (format, OC, IC), distinct contents, together larger than the last-level cache, and
+    the row scales; shared by the problems that differ only in their batch."""
 
-    def __init__(self, E, M, OC, IC, BS, device):
+    def __init__(self, E, M, OC, IC, device):
         import torch
         import fp6_llm_amd as fp6
         from fp6_llm_amd import quant, synth
 
-        self.E, self.M, self.OC, self.IC, self.BS = E, M, OC, IC, BS
-        self.splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC, EXPONENT=E, MANTISSA=M)
+        self.E, self.M, self.OC, self.IC, self.device = E, M, OC, IC, device
         nbytes = fp6.native_bytes(E, M, OC, IC)
         self.nbuf = int(max(2, min(128, POOL_BYTES // nbytes)))
         # distinct buffers, distinct contents: uniform random codes (every bit pattern is a valid weight)
@@ -98,6 +99,20 @@ class Problem:
         for i in range(self.nbuf):
             self.weights.append(torch.roll(base, shifts=257 * i) if i else base)
         self.scales = torch.from_numpy(synth.uniform_scales(2001, OC)).to(device)
+
+
+class Problem:
+    """Device buffers of one workload: a pool of native-layout weight buffers, scales, activations, output, workspace."""
+
+    def __init__(self, E, M, OC, IC, BS, device, pool=None):
+        import torch
+        import fp6_llm_amd as fp6
+        from fp6_llm_amd import synth
+
+        self.E, self.M, self.OC, self.IC, self.BS = E, M, OC, IC, BS
+        self.splitK = fp6.heuristic_splitk_mi355x(OC, BS, IC, EXPONENT=E, MANTISSA=M)
+        pool = pool or WeightPool(E, M, OC, IC, device)
+        self.nbuf, self.weights, self.scales = pool.nbuf, pool.weights, pool.scales
         self.x = torch.from_numpy(synth.activations(2001, BS, IC)).to(device)
         self.out = torch.empty((BS, OC), dtype=torch.float16, device=device)
         self.ws = torch.empty(self.splitK * BS * OC, dtype=torch.float32, device=device) if self.splitK > 1 else None
@@ -417,36 +432,86 @@ def run_workload(name, steps, warmup, device, with_fp16=True, with_warm=True, wi
     return res
 
 
-# One workload per benchmark configuration beyond the headline one, timed by the default run (`detail.configs`):
-# the MLP GEMMs of a 7B model at batch 32, the three GEMMs of a 70B layer at batch 32, and the 8192 x 8192 batch sweep's
-# ends and middle in both of the reference's formats.
-CONFIG_WORKLOADS = ["fp6_4096x4096_bs1", "fp6_4096x4096_bs16", "fp6_11008x4096_bs32", "fp6_4096x11008_bs32", "fp6_10240x8192_bs32",
-                    "fp6_28672x8192_bs32", "fp6_8192x28672_bs32", "fp6_8192x8192_bs1", "fp6_8192x8192_bs64", "fp6_8192x8192_bs512",
-                    "fp5_8192x8192_bs1", "fp5_8192x8192_bs64", "fp5_8192x8192_bs512"]
+# Every point of the benchmark configurations beyond the headline one, timed by the default run (`detail.configs`): 4096 x 4096 at
+# batch 1 and 16, the two MLP shapes of a 7B model at batch 8 and 32, the three GEMMs of a 70B layer at batch 32, and the
+# 8192 x 8192 sweep over ten batches in both of the reference's formats (the sweep of tests/python/run.sh:37-46).
+CONFIG_WORKLOADS = (["fp6_4096x4096_bs1", "fp6_4096x4096_bs16", "fp6_11008x4096_bs8", "fp6_11008x4096_bs32", "fp6_4096x11008_bs8", "fp6_4096x11008_bs32",
+                     "fp6_10240x8192_bs32", "fp6_28672x8192_bs32", "fp6_8192x28672_bs32"]
+                    + ["fp%d_8192x8192_bs%d" % (x, bs) for bs in (1, 2, 4, 8, 16, 32, 64, 128, 256, 512) for x in (6, 5)])
+
+
+class _Fp16Pool:
+    """fp16 weights of one shape rotating through 1 GiB like the FPx ones, for the FP16 library GEMM beside each workload."""
+
+    def __init__(self, OC, IC, device):
+        import torch
+        nb = OC * IC * 2
+        self.nbuf = int(max(2, min(64, POOL_BYTES // nb)))
+        self.ws = [torch.randn(OC, IC, dtype=torch.float16, device=device) for _ in range(self.nbuf)]
+
+
+def fp16_peak_tflops(device):
+    """One large square FP16 GEMM through torch (hipBLASLt): the MFMA rate a tuned library reaches on this GPU, to read the
+    large-batch figures against (the published peak of 2.5 PFLOP/s is not reached by any GEMM here)."""
+    import torch
+
+    n = 8192
+    a = torch.randn(n, n, dtype=torch.float16, device=device)
+    b = torch.randn(n, n, dtype=torch.float16, device=device)
+    for _ in range(5):
+        torch.matmul(a, b)
+    torch.cuda.synchronize()
+    best = None
+    for _ in range(3):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(10):
+            torch.matmul(a, b)
+        e1.record()
+        torch.cuda.synchronize()
+        t = e0.elapsed_time(e1) / 10 * 1e-3
+        best = t if best is None or t < best else best
+    return round(2.0 * n * n * n / best / 1e12, 1)
 
 
 def run_configs(device, budget_s):
-    """[{workload, us, hbm_frac | mfma_frac, fp16_us, speedup}] within a time budget (workloads that no longer fit are listed as skipped).
-    FP16 = torch F.linear (hipBLASLt) on fp16 weights of the same shape rotating the same way, same graph protocol."""
+    """[{workload, us, splitK, hbm_frac | mfma_frac, fp16_us, speedup}] within a time budget (workloads that no longer fit are listed
+    as skipped).  FP16 = torch F.linear (hipBLASLt) on fp16 weights of the same shape rotating the same way, same graph protocol;
+    workloads that share a weight matrix share its buffers, and an FP16 time is measured once per (shape, batch)."""
     import torch
 
     out, t0 = [], time.perf_counter()
+    pool, pool_key, f16pool, f16_key, f16_us = None, None, None, None, {}
     for name in CONFIG_WORKLOADS:
         if time.perf_counter() - t0 > budget_s:
             out.append({"workload": name, "skipped": "time budget"})
             continue
         E, M, OC, IC, BS = WORKLOADS[name]
+        if pool_key != (E, M, OC, IC):
+            pool = None
+            torch.cuda.empty_cache()
+            pool, pool_key = WeightPool(E, M, OC, IC, device), (E, M, OC, IC)
         big = OC * IC > 64e6
-        r = run_workload(name, 40 if big else 100, 5, device, with_warm=False, with_system_blas=False, with_floor=False)
-        entry = {"workload": name, "us": r["us_per_gemm"], "splitK": r["splitK"], "weight_GBps": r["weight_GBps"], "tflops": r["tflops"]}
+        steps = 40 if big else 100
+        prob = Problem(E, M, OC, IC, BS, device, pool)
+        us = time_steps(prob, steps, 5, cold=True)[1]
+        wb, flops = weight_bytes(E, M, OC, IC), 2.0 * OC * IC * BS
+        entry = {"workload": name, "us": round(us, 3), "splitK": prob.splitK, "weight_GBps": round(wb / us / 1e3, 1), "tflops": round(flops / us / 1e6, 2)}
         if BS >= 128:
-            entry["mfma_frac"] = r["mfma_frac"]
+            entry["mfma_frac"] = round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)
         else:
-            entry["hbm_frac"] = r["hbm_frac"]
-        entry["fp16_us"] = r["fp16_gemm_us"]
-        entry["speedup"] = r["speedup_vs_fp16"]
+            entry["hbm_frac"] = round(wb / us / 1e3 / HBM_PEAK_GBPS, 4)
+        if (OC, IC, BS) not in f16_us:
+            if f16_key != (OC, IC):
+                f16pool = None
+                torch.cuda.empty_cache()
+                f16pool, f16_key = _Fp16Pool(OC, IC, device), (OC, IC)
+            fw, x = f16pool, prob.x
+            f16_us[(OC, IC, BS)] = _time_fp16(lambda i: torch.nn.functional.linear(x, fw.ws[i % fw.nbuf]), steps, 5)
+        entry["fp16_us"] = round(f16_us[(OC, IC, BS)], 3)
+        entry["speedup"] = round(f16_us[(OC, IC, BS)] / us, 3)
         out.append(entry)
-        torch.cuda.empty_cache()
+        del prob
     return out
 
 
@@ -472,7 +537,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true",
                     help="skip the legs that run outside this process's GPU stream: the CPU path and the system-BLAS FP16 baseline (a child process)")
     ap.add_argument("--no-configs", action="store_true", help="skip detail.configs (one workload per benchmark configuration)")
-    ap.add_argument("--configs-budget", type=float, default=75.0, help="seconds the default run may spend on detail.configs")
+    ap.add_argument("--configs-budget", type=float, default=110.0, help="seconds the default run may spend on detail.configs")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="profiling aid: also run ten 64 MiB device-to-device copies, a kernel of known traffic to scale profiler byte counters by; "
                          "skips the FP16, CPU and per-configuration legs")
@@ -508,6 +573,7 @@ def main():
     res["launch_table"] = _lib.lib().fp6mi_tuning_info().decode()
     if not (args.no_configs or args.calibrate_copy):
         res["configs"] = run_configs(device, args.configs_budget)
+        res["fp16_peak_tflops_measured"] = fp16_peak_tflops(device)   # 8192^3 FP16 GEMM, torch/hipBLASLt
     compute_bound = BS >= 128
     line = {
         "metric": "weight bytes streamed per second by the FPx x FP16 GEMM (us/GEMM in ms_per_step)", "value": res["weight_GBps"], "unit": "GB/s",

@@ -277,6 +277,7 @@ def clear_caches():
     _native_cache.clear()
     if _ext is not None:
         _ext.clear_workspaces()
+        _ext.clear_twins()
 
 
 def _workspace(device, stream, nbytes):

@@ -351,7 +351,7 @@ const char *fp6mi_tuning_info(void)
         ;
 }
 
-int fp6mi_version(void) { return 132; } // 132: split-K reduction runs on the XCD that wrote the partial sums, every grid size gets XCD-contiguous tiles; 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
+int fp6mi_version(void) { return 133; } // 133: wave-specialized tile kernel (launch kind 2) for large batches; 132: split-K reduction runs on the XCD that wrote the partial sums, every grid size gets XCD-contiguous tiles; 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
 int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }

@@ -163,7 +163,15 @@ class Bench:
             with torch.cuda.graph(graph, stream=stream):
                 for i in range(self.iters):
                     launch(i)
+            # replays until about 8 ms have passed before any is timed: right after the idle spell of a capture the clocks are low,
+            # which costs a long kernel more than a short one
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
             graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            for _ in range(int(min(200, 8.0 / max(e0.elapsed_time(e1), 1e-3)))):
+                graph.replay()
             torch.cuda.synchronize()
             for _ in range(self.reps):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)

@@ -571,6 +571,31 @@ def test_scales_that_are_a_view_at_an_odd_half_offset(N):
     check_close(y.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "offset scales N=%d" % N)
 
 
+def test_cpp_torch_entry_points_on_reference_layout_weights():
+    """fp6_linear_forward_cuda / fp_eXmY_linear_forward_cuda of the torch extension (the reference's C++ names): same bits as the
+    Python functions of those names; the native twin follows the tensor (an in-place change of the weights is seen)."""
+    ext = fp6._ext
+    assert ext is not None, "fp6_llm_amd/_fp6mi_torch.so is built by python -m fp6_llm_amd.build"
+    for (E, M) in FORMATS:
+        OC, IC, N = 512, 1088, 9
+        raw, sc, x = synth.uniform_problem(860 + E + M, OC, IC, N, E, M)
+        packed = fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+        scd, xd = torch.from_numpy(sc).to(DEV), torch.from_numpy(x).to(DEV)
+        y = ext.linear_forward_eXmY_cuda(E, M, xd, packed, scd, 2)
+        assert torch.equal(y, fp6.linear_forward_eXmY_cuda(E, M, xd, packed, scd, 2))
+        check_close(y.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "C++ entry e%dm%d" % (E, M))
+        raw2, _, _ = synth.uniform_problem(870 + E + M, OC, IC, N, E, M)
+        packed.copy_(fp6.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw2)).to(DEV))   # same tensor object, new contents
+        y2 = ext.linear_forward_eXmY_cuda(E, M, xd, packed, scd, 1)
+        check_close(y2.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw2, sc, E, M), x), "C++ entry after an in-place update")
+    raw, sc, x = synth.uniform_problem(880, 256, 512, 3, 3, 2)
+    packed = fp6.weight_prepacking_cpu(torch.from_numpy(raw)).to(DEV)
+    y = ext.linear_forward_cuda(torch.from_numpy(x).to(DEV), packed, torch.from_numpy(sc).to(DEV), 1)
+    check_close(y.cpu().numpy(), oracle.gemm_f64(oracle.dequant(raw, sc, 3, 2), x), "fp6_linear_forward_cuda")
+    with pytest.raises(ValueError):
+        ext.linear_forward_cuda(torch.from_numpy(x).to(DEV), packed.cpu(), torch.from_numpy(sc).to(DEV), 1)   # weights must be on the GPU
+
+
 def test_module_forward():
     from fp6_llm_amd import module
     w = torch.from_numpy(synth.normal(31, (512, 1024))).float()

@@ -561,3 +561,31 @@ def test_launch_source_tells_measured_from_carried_over_from_rules():
     assert L.fp6mi_launch_source(3, 2, 4096, 8, 4096, 5) == 2          # a split the table does not hold
     assert L.fp6mi_launch_source(4, 3, 4096, 8, 4096, 1) == -1 and L.fp6mi_launch_source(3, 2, 100, 8, 4096, 1) == -2
     assert b"library version" in L.fp6mi_tuning_info()
+
+
+def test_cpp_torch_entry_points_carry_the_reference_names():
+    """The torch extension defines the reference's six C++ functions (fp6_llm/csrc/fp6_linear.cuh:50-90) and binds them under the
+    reference's Python names (fp6_llm/csrc/pybind.cpp:8-15); the CPU ones must give the oracle's bytes."""
+    ext = pytest.importorskip("fp6_llm_amd._fp6mi_torch")
+    for name in ("linear_forward_cuda", "weight_prepacking_cpu", "weight_dequant_cpu", "linear_forward_eXmY_cuda", "weight_prepacking_eXmY_cpu",
+                 "weight_dequant_eXmY_cpu"):
+        assert callable(getattr(ext, name))
+    header = open(os.path.join(os.path.dirname(fp6.__file__), "csrc", "fp6_linear_torch.h")).read()
+    for name in ("fp6_linear_forward_cuda", "fp_eXmY_linear_forward_cuda", "weight_matrix_prepacking_cpu", "weight_matrix_prepacking_fp_eXmY_cpu",
+                 "weight_matrix_dequant_cpu", "weight_matrix_dequant_fp_eXmY_cpu"):
+        assert name in header
+    for (E, M) in FORMATS:
+        raw, sc, _ = synth.uniform_problem(70 + E + M, 256, 320, 1, E, M)
+        packed = ext.weight_prepacking_eXmY_cpu(E, M, torch.from_numpy(raw))
+        assert packed.numpy().tobytes() == oracle.prepack(raw, E, M).tobytes()
+        deq = ext.weight_dequant_eXmY_cpu(E, M, torch.from_numpy(raw), torch.from_numpy(sc))
+        assert (deq.numpy().view(np.uint16) == oracle.dequant(raw, sc, E, M).view(np.uint16)).all()
+    raw, sc, _ = synth.uniform_problem(71, 256, 320, 1, 3, 2)
+    assert torch.equal(ext.weight_prepacking_cpu(torch.from_numpy(raw)), fp6.weight_prepacking_cpu(torch.from_numpy(raw)))
+    assert torch.equal(ext.weight_dequant_cpu(torch.from_numpy(raw), torch.from_numpy(sc)), fp6.weight_dequant_cpu(torch.from_numpy(raw), torch.from_numpy(sc)))
+    with pytest.raises(ValueError):
+        ext.weight_prepacking_cpu(torch.zeros((100, 12), dtype=torch.int32))           # OC % 256 (the reference asserts)
+    with pytest.raises(ValueError):
+        ext.weight_prepacking_eXmY_cpu(4, 3, torch.zeros((256, 16), dtype=torch.int32))  # a format nobody has
+    with pytest.raises(ValueError):
+        ext.weight_dequant_cpu(torch.zeros((256, 12), dtype=torch.int32), torch.zeros(255, dtype=torch.float16))
