@@ -3,7 +3,8 @@
 // exports one table of entry functions (fp6mi::FormatOps) that the C ABI in fp6mi_api.hip dispatches to.
 //
 // Roles taken over from the reference (usyd-fsalab/fp6_llm, paths relative to it):
-//   gemm_stream   <- QUANT_GEMM_Kernel        fp6_llm/csrc/include/kernel_matmul.cuh:29-191
+//   gemm_stream, gemm_tile, gemm_ws <- QUANT_GEMM_Kernel   fp6_llm/csrc/include/kernel_matmul.cuh:29-191
+//                    (small batches / batches above 16 / large batches: three organisations of the same GEMM)
 //   splitk_reduce <- SplitK_Reduction         fp6_llm/csrc/include/kernel_reduction.cuh:28-47   (in fp6mi_api.hip)
 //   launchers     <- fpx_linear_kernel        fp6_llm/csrc/fp6_linear.cu:44-102
 // The design is not a translation: weights use the native layout described in fp6mi_host.cpp, go from HBM straight

@@ -99,8 +99,10 @@ def _all_candidates(OC, IC, BS, bits=6):
         cfgs = STREAM_SMALL
     else:
         cfgs = [c for c in TILE if (c[1] * 16 < 2 * BS + 16 or c[1] == 2) and (BS <= 512 or c[1] >= 4)]
-        if BS <= 32:
-            cfgs = cfgs + STREAM_WIDE
+        if BS <= 64:    # the stream kernel over several column blocks (each re-reads the weights, out of L2): wins on small M, where
+            cfgs = cfgs + STREAM_WIDE + STREAM_SMALL   # a tile kernel would have to split K to fill the chip (4096 x 4096 batch 24-64)
+        elif BS <= 128 and OC <= 2560:   # the same for matrices of so few rows that even at batch 128 no tile shape fills the chip
+            cfgs = cfgs + STREAM_WIDE + STREAM_SMALL
         if BS >= 96:    # the wave-specialized tiles pay from about 128 columns up (256 x 64 from 256 up on 8192 x 8192)
             cfgs = cfgs + [c for c in COMPILED_WS if c[1] * 16 <= BS]
     units = (IC + 255) // 256
