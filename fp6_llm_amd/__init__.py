@@ -281,6 +281,10 @@ def clear_caches():
 
 
 def _workspace(device, stream, nbytes):
+    if torch.cuda.is_current_stream_capturing():
+        # memory allocated now belongs to the graph being recorded: hand it to this call only (the graph keeps it for its
+        # replays) and remember nothing, or a later eager call would share scratch memory with the graph's replays
+        return torch.empty((nbytes + 3) // 4, dtype=torch.float32, device=device)
     key = (device.index, stream)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() * 4 < nbytes:

@@ -26,6 +26,11 @@ std::map<std::pair<int, void *>, at::Tensor>       g_workspaces; // (device, str
 
 at::Tensor workspace_for(const at::Device &dev, void *stream, int64_t floats)
 {
+    // Under stream capture the memory belongs to the graph being recorded: this call gets a tensor of its own (the graph keeps
+    // the memory for its replays) and nothing is remembered, or a later eager call would share scratch with those replays.
+    hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(static_cast<hipStream_t>(stream), &capture) == hipSuccess && capture != hipStreamCaptureStatusNone)
+        return at::empty({ floats }, at::TensorOptions().dtype(at::kFloat).device(dev));
     std::lock_guard<std::mutex> lock(g_ws_mutex);
     auto                        key = std::make_pair((int)dev.index(), stream);
     auto                        it = g_workspaces.find(key);

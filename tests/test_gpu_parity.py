@@ -524,6 +524,42 @@ def test_graph_capture_replays_match_eager():
             assert torch.equal(out, eager), (N, splitK, rep)
 
 
+def test_split_k_workspace_first_needed_under_capture_is_not_shared_with_eager_calls():
+    """A split-K call without a caller's workspace, first made while its stream is being captured: the scratch it gets
+    belongs to the graph.  Eager split-K calls made afterwards (same stream object, other streams) must not be handed that
+    memory: replays interleaved with eager calls on another stream all equal the plain results."""
+    E, M = 3, 2
+    OC, IC, N, splitK = 512, 2048, 40, 4
+    raw, sc, _ = synth.uniform_problem(870, OC, IC, 1, E, M)
+    native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+    scd = torch.from_numpy(sc).to(DEV)
+    fp6.clear_caches()
+    x = torch.zeros((N, IC), dtype=torch.float16, device=DEV)
+    out = torch.empty((N, OC), dtype=torch.float16, device=DEV)
+    s, other = torch.cuda.Stream(), torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g, stream=s):
+            fp6.linear_forward_native(E, M, x, native, scd, OC, splitK, out=out)
+    assert not fp6._workspaces, "scratch allocated under capture was remembered"
+    for rep in range(3):
+        xin = torch.from_numpy(synth.activations(880 + rep, N, IC)).to(DEV)
+        plain = fp6.linear_forward_native(E, M, xin, native, scd, OC, 1)
+        torch.cuda.synchronize()
+        x.copy_(xin)
+        torch.cuda.synchronize()
+        with torch.cuda.stream(s):
+            g.replay()
+        with torch.cuda.stream(other):
+            eager = fp6.linear_forward_native(E, M, xin, native, scd, OC, splitK)
+        with torch.cuda.stream(s):
+            eager_same = fp6.linear_forward_native(E, M, xin, native, scd, OC, splitK)
+        torch.cuda.synchronize()
+        check_close(out.cpu().numpy(), plain.float().cpu().numpy(), "replay %d" % rep)
+        assert torch.equal(eager, out) and torch.equal(eager_same, out), rep
+
+
 def test_reference_named_api_first_use_under_capture_then_eager_before_replay():
     """linear_forward_cuda on reference-layout weights whose FIRST use is inside a stream capture: the conversion is only
     recorded there, so nothing may be remembered from it.  An eager call before the first replay must convert for itself and
