@@ -147,7 +147,8 @@ const TuneEntry kTune[] = {
 #include "fp6mi_tuning.inc"
 };
 
-inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && M % (16u * c.rt * (c.kind >= 1 ? c.wr : 1u)) == 0; }
+// (the stream kernel takes any number of row tiles per workgroup for any M: its last workgroup may hold fewer)
+inline bool cfg_fits(const TuneCfg &c, size_t M) { return c.kind != 255 && (c.kind == 0 || M % (16u * c.rt * c.wr) == 0); }
 
 // What the table says about a problem that need not be in it: per splitK the shape expected to be fastest and its expected
 // time.  The batch is rounded UP to a measured batch of the same kernel family (a shape's cost steps at column-tile
@@ -176,7 +177,7 @@ const std::vector<TuneGroup> &tune_groups()
 inline double rounds_on_chip(const TuneCfg &c, size_t M, size_t N, int splitK)
 {
     const size_t TM = (size_t)(c.kind >= 1 ? c.wr : 1) * c.rt * 16, TN = (size_t)c.nt * 16;
-    const double wgs = (double)(M / TM) * (double)((N + TN - 1) / TN) * splitK;
+    const double wgs = (double)((M + TM - 1) / TM) * (double)((N + TN - 1) / TN) * splitK;
     // tile kernel: one workgroup per CU, two for four-wavefront workgroups.  Stream kernel: several workgroups share a CU, but
     // they share its memory pipeline too, so what counts is the largest number of workgroups any CU is given.
     const double slots = 256.0 * (c.kind == 1 && c.wr * c.wk <= 4 ? 2 : 1);
@@ -266,18 +267,22 @@ inline LaunchCfg pick_cfg(int xbits, size_t M, size_t N, size_t K, int splitK, i
             else if (per_cu < 3.125) { c.rt = 1; c.wk = 4; }
             else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
             else                     { c.rt = 2; c.wk = 8; }
-        } else if (N <= 8) {
-            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
-            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 8; }
-            else if (per_cu < 3.125) { c.rt = 4; c.wk = 8; }
-            else if (per_cu < 5.5)   { c.rt = 2; c.wk = 4; }
-            else                     { c.rt = 4; c.wk = 4; }
         } else {
-            if (per_cu < 1.5)        { c.rt = 1; c.wk = 8; }
-            else if (per_cu < 2.5)   { c.rt = 2; c.wk = 4; }
-            else                     { c.rt = 4; c.wk = 4; }
+            // Batches 5..16: every row tile a workgroup adds re-uses its activation registers, and a CU is done when its last
+            // workgroup is, so give each CU its share of the row tiles in as few workgroups as hold them (at most eight tiles):
+            // cost of rt tiles per workgroup = rounds of the 256 CUs x rt.  10240, 11008 and 12288 rows take 3, 17920 and 19968
+            // rows 5, 22016 rows 6, 28672 rows 7 (measured: 5-20 % better than the power of two next to them).  Ties go to the
+            // larger workgroup (12288 rows: three tiles at once beat three workgroups of one by 7 %).
+            int    best = 1;
+            size_t best_cost = ~(size_t)0;
+            for (int rt = 1; rt <= 8; rt++) {
+                const size_t wgs = (tiles + rt - 1) / rt * splitK, cost = (wgs + cus - 1) / cus * rt;
+                if (cost <= best_cost) best = rt, best_cost = cost;
+            }
+            c.rt = best;
+            c.wk = best >= 5 || (best == 4 && N > 8) ? 4 : 8;
         }
-        while (c.rt > 1 && tiles % c.rt) c.rt /= 2;
+        while ((c.rt == 2 || c.rt == 4 || c.rt == 8) && tiles % c.rt) c.rt /= 2; // (the other counts need not divide: the last workgroup holds the rest)
         const int cap = per_split > 8 ? 16 : per_split > 4 ? 8 : 4; // no more wavefronts than K blocks to hand out
         if (c.wk > cap) c.wk = cap;
         if (c.rt == 4 && c.wk == 16) c.wk = 8; // not compiled: 16 wavefronts leave too few registers for four row tiles
@@ -295,7 +300,7 @@ int linear_native(const fp6mi::FormatOps &ops, hipStream_t st, const void *W, co
                   int splitK, const LaunchCfg *forced)
 {
     LaunchCfg c = forced ? *forced : pick_cfg(ops.bits, M, N, K, splitK, current_device_cus());
-    if (c.kind == 0 && (M / 16) % c.rt) return FP6MI_ERR_SHAPE;
+    if (c.kind == 0 && !(c.rt & (c.rt - 1)) && (M / 16) % c.rt) return FP6MI_ERR_SHAPE; // (3, 5, 6, 7 tiles per workgroup end in a workgroup with fewer)
     int rc = ops.gemm(c, st, W, sc, gexp, B, C, ws, M, N, K, splitK);
     if (rc != 0) return rc;
     if (splitK > 1) {
@@ -351,7 +356,7 @@ const char *fp6mi_tuning_info(void)
         ;
 }
 
-int fp6mi_version(void) { return 133; } // 133: wave-specialized tile kernel (launch kind 2) for large batches; 132: split-K reduction runs on the XCD that wrote the partial sums, every grid size gets XCD-contiguous tiles; 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
+int fp6mi_version(void) { return 134; } // 134: three row tiles per workgroup in the small-batch kernel (any M: the last workgroup takes what is left), no other kernel changed; 133: wave-specialized tile kernel (launch kind 2) for large batches; 132: split-K reduction runs on the XCD that wrote the partial sums, every grid size gets XCD-contiguous tiles; 131: tile kernel stores through LDS; 130: small-batch kernel loads activations as whole rows and turns them into operand order through LDS
 
 int fp6mi_prepack_ref(int E, int Mb, void *packed, const void *raw, size_t M, size_t K) { return fp6mi::prepack_ref(E, Mb, packed, raw, M, K); }
 int fp6mi_unpack_ref(int E, int Mb, void *raw, const void *packed, size_t M, size_t K) { return fp6mi::unpack_ref(E, Mb, raw, packed, M, K); }

@@ -219,6 +219,12 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
     const size_t   tile_stride = (size_t)units * Fmt<FM>::block_bytes;
     const uint8_t *wgroup = W + (size_t)R0 * tile_stride;
     const uint8_t *ggroup = GS ? gexp + (size_t)R0 * units * 32 : nullptr;
+    // M is a multiple of 256, so 1, 2, 4 and 8 row tiles per workgroup divide its M/16 row tiles; 3, 5, 6 and 7 need not, and
+    // the last workgroup then holds fewer.  Its missing tiles stand in as copies of its last real one (same loads, same arithmetic,
+    // nothing stored): rlast is the largest r that names a real tile.
+    constexpr bool kRagged = (RT & (RT - 1)) != 0;
+    const uint32_t rlast = kRagged && R0 + RT > (M >> 4) ? (M >> 4) - 1 - R0 : RT - 1;
+    auto           real = [&](int r) -> uint32_t { return kRagged && (uint32_t)r > rlast ? rlast : (uint32_t)r; };
 
     v4f acc[RT][NT];
 #pragma unroll
@@ -233,7 +239,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 #pragma unroll
     for (int j = 0; j < kOutPerThread; j++) {
         int e = threadIdx.x + j * WAVES * kWave;
-        my_scale[j] = scales[(R0 + (e < RT * NT * 256 ? (e >> 8) / NT : 0)) * 16 + (e & 15)];
+        my_scale[j] = scales[(R0 + real(e < RT * NT * 256 ? (e >> 8) / NT : 0)) * 16 + (e & 15)];
     }
 
     const uint32_t ncols = N - nbase;              // batch columns of this column block that exist (the launcher made sure of >= 1)
@@ -276,7 +282,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
             v4u            xv[LOADS];
             auto           wpart = [&](int i) {
                 const int r = i / kWParts, part = i % kWParts;
-                load_wfrag_part<FM>(cur.w[r], wgroup + r * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
+                load_wfrag_part<FM>(cur.w[r], wgroup + real(r) * tile_stride + (size_t)u * Fmt<FM>::block_bytes, lane, part);
             };
 #pragma unroll
             for (int i = 0; i < kWBeforeX; i++) wpart(i);
@@ -300,7 +306,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 #pragma unroll
             for (int i = kWBeforeX; i < RT * kWParts; i++) wpart(i);
 #pragma unroll
-            for (int r = 0; r < RT; r++) cur.g[r] = load_group_exps<GS>(ggroup, (size_t)r * units + u, lane);
+            for (int r = 0; r < RT; r++) cur.g[r] = load_group_exps<GS>(ggroup, (size_t)real(r) * units + u, lane);
             __builtin_amdgcn_sched_barrier(0); // keep every load of the block issued before anything waits
             v8h x[8][NT];
             if constexpr (MODE == 0) {
@@ -375,7 +381,7 @@ __global__ __launch_bounds__(WAVES *kWave) void gemm_stream(const uint8_t *__res
 #pragma unroll
         for (int w = 0; w < WAVES; w++) sum += *reinterpret_cast<const float *>(lds + w * wave_bytes + rt * 1024 + idx * 4);
         uint32_t ng = nbase + 16 * t + n, mg = (R0 + r) * 16 + mm;
-        if (ng < N) {
+        if (ng < N && (!kRagged || (uint32_t)r <= rlast)) {
             float v = sum * ((float)my_scale[j] * Fmt<FM>::post_scale);
             if constexpr (!SPLIT)
                 C[(size_t)ng * M + mg] = (half_t)v;
@@ -1207,7 +1213,7 @@ int launch_stream(hipStream_t st, const void *W, const void *sc, const void *gex
     constexpr size_t kMaxLds = (size_t)WAVES * stream_wave_bytes(16 * NT, RT, NT);
     static_assert(kMaxLds <= 160 * 1024, "the wavefronts' activation rows do not fit in LDS");
     uint32_t     units = (uint32_t)((K + 255) / 256);
-    dim3         grid((uint32_t)(M / (16 * RT)), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
+    dim3         grid((uint32_t)((M / 16 + RT - 1) / RT), (uint32_t)splitK, (uint32_t)((N + 16 * NT - 1) / (16 * NT)));
     const size_t lds_bytes = NT == 1 && N <= 8 ? (size_t)WAVES * stream_wave_bytes(8, RT, NT) : kMaxLds;
     auto         go = [&](auto kernel_c) -> int {
         constexpr auto kernel = decltype(kernel_c)::value;
@@ -1280,9 +1286,13 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
     if (c.nt == NT && c.rt == RT && c.wk == WV && c.wr == 1) return launch_stream<FM, GS, NT, RT, WV>(st, W, sc, gexp, B, C, ws, M, N, K, splitK);
         FP6MI_CASE(1, 1, 4) FP6MI_CASE(1, 1, 8) FP6MI_CASE(1, 1, 16)
         FP6MI_CASE(1, 2, 4) FP6MI_CASE(1, 2, 8) FP6MI_CASE(1, 2, 16)
+        FP6MI_CASE(1, 3, 4) FP6MI_CASE(1, 3, 8)
         FP6MI_CASE(1, 4, 4) FP6MI_CASE(1, 4, 8)
+        FP6MI_CASE(1, 5, 4) FP6MI_CASE(1, 5, 8) FP6MI_CASE(1, 6, 4) FP6MI_CASE(1, 6, 8) FP6MI_CASE(1, 7, 4) FP6MI_CASE(1, 8, 4)
         FP6MI_CASE(2, 1, 4) FP6MI_CASE(2, 1, 8)
         FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
+        FP6MI_CASE(2, 3, 4) FP6MI_CASE(2, 3, 8)
+        FP6MI_CASE(2, 4, 4) FP6MI_CASE(2, 4, 8)
 #undef FP6MI_CASE
     } else if (c.kind == 1) {
 #define FP6MI_CASE(NT, RT, WR, WK) \

@@ -25,8 +25,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 INC_PATH = os.path.join(HERE, "csrc", "fp6mi_tuning.inc")
 
 # (kind, n_tiles, row_tiles, row_waves, k_waves); kind 0 = stream kernel (batch <= 16 per n_tile), 1 = tile kernel, 2 = wave-specialized tile kernel
-STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 4) for wk in (4, 8, 16) if (rt, wk) != (4, 16)]
-STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4)]                      # two 16-column tiles per workgroup, batches 17..32
+STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 3, 4, 5, 6, 7, 8) for wk in (4, 8, 16) if wk == 4 or (wk == 8 and rt <= 6) or rt <= 2]
+STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 3, 1, 4), (0, 2, 3, 1, 8), (0, 2, 4, 1, 4), (0, 2, 4, 1, 8)]   # two 16-column tiles per workgroup, batches 17..32
 TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
         (1, 8, 2, 8, 1)]
 SPLITS = (1, 2, 3, 4, 6, 8)      # 3 and 6 fill 256 CUs where 80 or 40 row blocks leave a power of two short (M = 10240, 5120)
@@ -35,8 +35,9 @@ FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit
 # every shape compiled into the library (FP6MI_CASE tables of csrc/fp6mi_gemm.hip, the same for every format); the candidates above are the ones that
 # ever came within 3 % of the best in exhaustive sweeps
 COMPILED_STREAM = [(0, nt, rt, 1, wk) for (nt, rt, wk) in
-                   [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 4, 4), (1, 4, 8), (2, 1, 4), (2, 1, 8), (2, 2, 4),
-                    (2, 2, 8)]]
+                   [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 3, 4), (1, 3, 8), (1, 4, 4), (1, 4, 8), (1, 5, 4),
+                    (1, 5, 8), (1, 6, 4), (1, 6, 8), (1, 7, 4), (1, 8, 4), (2, 1, 4), (2, 1, 8), (2, 2, 4), (2, 2, 8), (2, 3, 4), (2, 3, 8),
+                    (2, 4, 4), (2, 4, 8)]]
 COMPILED_TILE = [(1,) + c for c in
                  [(2, 1, 4, 4), (2, 2, 4, 4), (2, 2, 4, 2), (2, 2, 4, 1), (2, 4, 4, 1), (2, 4, 4, 2), (4, 2, 4, 2), (4, 2, 4, 1), (4, 4, 4, 1),
                   (4, 4, 2, 1), (4, 4, 2, 2), (8, 2, 4, 1), (8, 2, 2, 1), (4, 2, 8, 1), (4, 2, 8, 2), (2, 2, 8, 1), (2, 2, 8, 2), (8, 2, 8, 1),
@@ -84,10 +85,13 @@ def tile_rows(cfg):
 KIND_NAMES = ("stream", "tile", "ws")
 
 
-def candidates(OC, IC, BS, kinds=None, splits=None, bits=6):
-    """(shape, splitK) pairs worth measuring; `kinds` ("stream", "tile", "ws") and `splits` narrow the list for a partial sweep."""
+def candidates(OC, IC, BS, kinds=None, splits=None, bits=6, shapes=None):
+    """(shape, splitK) pairs worth measuring; `kinds` ("stream", "tile", "ws"), `splits` and `shapes` (a set of shape tuples)
+    narrow the list for a partial sweep."""
     for cfg, sk in _all_candidates(OC, IC, BS, bits):
         if kinds and KIND_NAMES[cfg[0]] not in kinds:
+            continue
+        if shapes and tuple(cfg) not in shapes:
             continue
         if splits and sk not in splits:
             continue
@@ -107,7 +111,7 @@ def _all_candidates(OC, IC, BS, bits=6):
             cfgs = cfgs + [c for c in COMPILED_WS if c[1] * 16 <= BS]
     units = (IC + 255) // 256
     for cfg in cfgs:
-        if OC % tile_rows(cfg):
+        if OC % tile_rows(cfg) and cfg[0] != 0:   # (the stream kernel takes any number of row tiles per workgroup: the last one holds the rest)
             continue
         for sk in SPLITS:
             if sk > units or (cfg[0] == 0 and sk > 1 and OC > 4096):   # the stream kernel splits K inside the workgroup already
@@ -198,6 +202,7 @@ def sweep(args):
         problems = [(OC, IC) for OC in Ms for IC in Ks]
     kinds = set(args.kinds.split(",")) if args.kinds else None
     splits = set(int(v) for v in args.splits.split(",")) if args.splits else None
+    shapes = set(tuple(int(v) for v in sh.split(".")) for sh in args.shapes.split(",")) if args.shapes else None
     bench = Bench(args.iters, args.reps)
     os.makedirs(os.path.dirname(os.path.abspath(args.out)), exist_ok=True)
     with open(args.out, "a" if args.append else "w") as f:
@@ -207,12 +212,16 @@ def sweep(args):
                     continue
                 for BS in Ns:
                     best = {}
-                    for cfg, sk in candidates(OC, IC, BS, kinds, splits, args.format):
+                    for cfg, sk in candidates(OC, IC, BS, kinds, splits, args.format, shapes):
                         t = bench(E, M, OC, IC, BS, cfg, sk)
                         if t is not None and (str(sk) not in best or t < best[str(sk)][1]):
                             best[str(sk)] = [list(cfg), round(t, 3)]
                     row = {"E": E, "M": M, "OC": OC, "IC": IC, "BS": BS, "best": best, "lib": bench.lib_version, "rocm": bench.rocm}
-                    if kinds or splits:   # a partial row: `merge` folds it into a full one
+                    if shapes:            # new shapes only: nothing measured before is out of date, `merge` keeps the faster entry
+                        if not best:
+                            continue
+                        row["partial"] = {"kinds": [], "splits": []}
+                    elif kinds or splits:   # a partial row: `merge` folds it into a full one
                         row["partial"] = {"kinds": sorted(kinds) if kinds else list(KIND_NAMES), "splits": sorted(splits) if splits else list(SPLITS)}
                     f.write(json.dumps(row) + "\n")
                     f.flush()
@@ -312,6 +321,7 @@ def main(argv=None):
     s.add_argument("--pairs", default="", help="OCxIC,OCxIC,... instead of the m x k grid, or `models` for the built-in list of layer shapes")
     s.add_argument("--kinds", default="", help="stream, tile, ws (comma-separated): measure only these kernels' shapes (the rows are partial: see merge)")
     s.add_argument("--splits", default="", help="measure only these splitK values (the rows are partial: see merge)")
+    s.add_argument("--shapes", default="", help="measure only these shapes, kind.nt.rt.wr.wk,... (shapes added to the library: merge keeps the faster of old and new)")
     s.add_argument("--iters", type=int, default=30)
     s.add_argument("--reps", type=int, default=5)
     s.set_defaults(fn=sweep)

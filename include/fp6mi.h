@@ -132,7 +132,8 @@ int fp6mi_linear_stateless(int E, int Mbits, void *stream, const void *W_ref, co
 
 /* Tuning hook: the same GEMM with the launch shape chosen by the caller instead of the built-in selection
  * (no counterpart in the reference, whose TilingConfig is picked inside fpx_linear_kernel, fp6_linear.cu:61-81).
- * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup),
+ * kind 0 = stream kernel (row_waves must be 1, k_waves in {4,8,16} wavefronts split K inside the workgroup; row_tiles = 1..8, where
+ *          3, 5, 6 and 7 need not divide M/16: the last workgroup holds the tiles that are left),
  * kind 1 = tile kernel (row_waves x k_waves wavefronts, activations staged in LDS),
  * kind 2 = wave-specialized tile kernel (row_waves arithmetic wavefronts; k_waves = 4 loading wavefronts that move weights and
  *          activations into LDS for them);

@@ -149,6 +149,43 @@ def test_every_launch_shape(E, M, cfg):
 
 
 @pytest.mark.parametrize("E,M", FORMATS)
+@pytest.mark.parametrize("cfg", [c for c in STREAM_SHAPES if c[2] in (3, 5, 6, 7)])
+def test_stream_kernel_row_tile_counts_with_a_short_last_workgroup(E, M, cfg):
+    """Three, five, six or seven row tiles per workgroup do not divide every M: 256 rows are 16 tiles (with three per workgroup
+    the sixth workgroup holds one), 512 rows 32 (the eleventh holds two), 768 rows 48 (none short with three, three left for the
+    tenth with five).  Results equal the oracle's, with and without split-K and group exponents, and nothing is written past
+    the end of the output or of the workspace."""
+    print("case row tiles per workgroup", E, M, cfg, flush=True)
+    L = _lib.lib()
+    IC, N = 1344, 16 * cfg[1] - 5
+    stream = torch.cuda.current_stream().cuda_stream
+    for OC in (256, 512, 768):
+        codes, sc, ex = quant.quantize_groupwise(_grouped_weights(OC + IC + sum(cfg), OC, IC), E, M)
+        raw = quant.pack_raw(codes, E, M)
+        native = fp6.weight_prepacking_native_cpu(E, M, torch.from_numpy(raw)).to(DEV)
+        gexp = fp6.pack_group_exps(torch.from_numpy(ex), OC, IC).to(DEV)
+        scd = torch.from_numpy(sc).to(DEV)
+        x = synth.activations(OC + 7, N, IC)
+        xd = torch.from_numpy(x).to(DEV)
+        refs = {False: oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), True: oracle.gemm_f64(oracle.dequant_grouped_from_definition(codes, sc, ex, E, M), x)}
+        for grouped in (False, True):
+            for splitK in (1, 2):
+                out = torch.full((N * OC + 4096,), 777.0, dtype=torch.float16, device=DEV)
+                ws = torch.full((splitK * N * OC + 4096,), 777.0, dtype=torch.float32, device=DEV)
+                if grouped:
+                    rc = L.fp6mi_linear_native_grouped_cfg(E, M, stream, native.data_ptr(), scd.data_ptr(), gexp.data_ptr(), xd.data_ptr(), out.data_ptr(),
+                                                           OC, N, IC, ws.data_ptr(), splitK, *cfg)
+                else:
+                    rc = L.fp6mi_linear_native_cfg(E, M, stream, native.data_ptr(), scd.data_ptr(), xd.data_ptr(), out.data_ptr(), OC, N, IC, ws.data_ptr(),
+                                                   splitK, *cfg)
+                assert rc == 0, rc
+                torch.cuda.synchronize()
+                y = out[:N * OC].view(N, OC).float().cpu().numpy()
+                check_close(y, refs[grouped], "cfg %s OC %d grouped %s splitK %d" % (cfg, OC, grouped, splitK))
+                assert (out[N * OC:] == 777.0).all() and (ws[splitK * N * OC:] == 777.0).all(), "written past the end"
+
+
+@pytest.mark.parametrize("E,M", FORMATS)
 @pytest.mark.parametrize("cfg", WS_SHAPES)
 def test_wave_specialized_kernel_edges(E, M, cfg):
     """The kernel whose loading wavefronts fill LDS rings for its arithmetic wavefronts, where its bookkeeping is thinnest: a K

@@ -243,14 +243,14 @@ def test_measured_table_holds_only_compiled_shapes_and_query_launch_follows_it()
             if v[0] == 255:
                 continue
             assert v[:5] in compiled, (xb, OC, IC, BS, v)
-            assert OC % tune.tile_rows(v[:5]) == 0
+            assert v[0] == 0 or OC % tune.tile_rows(v[:5]) == 0      # (the stream kernel's last workgroup holds what is left of the row tiles)
             assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, tune.SPLITS[i], shape) == 0
             assert tuple(shape) == v[:5], (xb, OC, IC, BS, tune.SPLITS[i], tuple(shape), v)
     # any legal problem gets a compiled shape that divides its rows, measured neighbour or not
     for (OC, IC, BS, sk) in [(256, 64, 1, 1), (768, 1088, 3, 2), (4352, 4160, 8, 1), (9984, 3008, 40, 3), (65536, 16384, 700, 1), (512, 64, 17, 1)]:
         for (E, Mb) in FORMATS:
             assert L.fp6mi_query_launch(E, Mb, OC, BS, IC, sk, shape) == 0
-            assert tuple(shape) in compiled and OC % tune.tile_rows(tuple(shape)) == 0, (OC, IC, BS, sk, tuple(shape))
+            assert tuple(shape) in compiled and (shape[0] == 0 or OC % tune.tile_rows(tuple(shape)) == 0), (OC, IC, BS, sk, tuple(shape))
     assert L.fp6mi_query_launch(3, 2, 100, 1, 64, 1, shape) == -2 and L.fp6mi_query_launch(4, 3, 256, 1, 64, 1, shape) == -1
 
 
@@ -492,7 +492,8 @@ def test_tuner_candidates_and_table_emission(tmp_path, monkeypatch):
         cands = list(tune.candidates(OC, IC, BS))
         assert cands, (OC, IC, BS)
         for cfg, sk in cands:
-            assert cfg in compiled and OC % tune.tile_rows(cfg) == 0 and 1 <= sk <= (IC + 255) // 256
+            ragged = cfg[0] == 0                       # the stream kernel's last workgroup holds what is left of the row tiles
+            assert cfg in compiled and (ragged or OC % tune.tile_rows(cfg) == 0) and 1 <= sk <= (IC + 255) // 256
             assert cfg[0] != 0 or BS <= 64 or (BS <= 128 and OC <= 2560)     # the stream kernel is a candidate up to four column blocks, eight on short matrices
             assert cfg[0] == 0 or BS > 16
     src = tmp_path / "t.jsonl"
