@@ -59,18 +59,19 @@ HEADLINE = "fp6_4096x4096_bs8"
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, each scaled by what the same counter reads
 # for a 64 MiB device copy (`--calibrate-copy`); the runs and readings are in profiles/gemm_*_<workload>.md.
 MEASURED_TRAFFIC_BYTES = {   # workload: bytes per launch of the GEMM kernel, and fp6mi_version() of the library that was profiled
-    "fp4_8192x8192_bs8": {"bytes": 34856037, "lib_version": 133},
-    "fp5_8192x8192_bs1": {"bytes": 42240541, "lib_version": 133},
-    "fp5_8192x8192_bs64": {"bytes": 58867404, "lib_version": 133},
-    "fp5_8192x8192_bs8": {"bytes": 43259104, "lib_version": 133},
-    "fp6_10240x8192_bs32": {"bytes": 71144412, "lib_version": 133},
-    "fp6_11008x4096_bs32": {"bytes": 41678487, "lib_version": 133},
-    "fp6_28672x8192_bs32": {"bytes": 182283423, "lib_version": 133},
-    "fp6_4096x4096_bs8": {"bytes": 13294045, "lib_version": 133},
-    "fp6_8192x8192_bs1": {"bytes": 50633372, "lib_version": 133},
-    "fp6_8192x8192_bs512": {"bytes": 125938394, "lib_version": 133},
-    "fp6_8192x8192_bs64": {"bytes": 69144949, "lib_version": 133},
-    "fp6_8192x8192_bs8": {"bytes": 51631462, "lib_version": 133},
+    "fp4_8192x8192_bs8": {"bytes": 34856037, "lib_version": 134},
+    "fp5_8192x8192_bs1": {"bytes": 42218021, "lib_version": 134},
+    "fp5_8192x8192_bs64": {"bytes": 58875593, "lib_version": 134},
+    "fp5_8192x8192_bs8": {"bytes": 43262175, "lib_version": 134},
+    "fp6_10240x8192_bs32": {"bytes": 75087832, "lib_version": 134},
+    "fp6_11008x4096_bs32": {"bytes": 36735643, "lib_version": 134},
+    "fp6_11008x4096_bs8": {"bytes": 34670774, "lib_version": 134},
+    "fp6_28672x8192_bs32": {"bytes": 182287518, "lib_version": 134},
+    "fp6_4096x4096_bs8": {"bytes": 13288927, "lib_version": 134},
+    "fp6_8192x8192_bs1": {"bytes": 50623135, "lib_version": 134},
+    "fp6_8192x8192_bs512": {"bytes": 125930205, "lib_version": 134},
+    "fp6_8192x8192_bs64": {"bytes": 67853755, "lib_version": 134},
+    "fp6_8192x8192_bs8": {"bytes": 51635556, "lib_version": 134},
 }
 
 
