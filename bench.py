@@ -66,7 +66,7 @@ MEASURED_TRAFFIC_BYTES = {   # workload: bytes per launch of the GEMM kernel, an
     "fp6_10240x8192_bs32": {"bytes": 75087832, "lib_version": 134},
     "fp6_11008x4096_bs32": {"bytes": 36735643, "lib_version": 134},
     "fp6_11008x4096_bs8": {"bytes": 34670774, "lib_version": 134},
-    "fp6_28672x8192_bs32": {"bytes": 182287518, "lib_version": 134},
+    "fp6_28672x8192_bs32": {"bytes": 182364291, "lib_version": 134},
     "fp6_4096x4096_bs8": {"bytes": 13288927, "lib_version": 134},
     "fp6_8192x8192_bs1": {"bytes": 50623135, "lib_version": 134},
     "fp6_8192x8192_bs512": {"bytes": 125930205, "lib_version": 134},

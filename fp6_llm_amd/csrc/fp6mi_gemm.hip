@@ -1293,6 +1293,7 @@ int launch_cfg(const LaunchCfg &c, hipStream_t st, const void *W, const void *sc
         FP6MI_CASE(2, 2, 4) FP6MI_CASE(2, 2, 8)
         FP6MI_CASE(2, 3, 4) FP6MI_CASE(2, 3, 8)
         FP6MI_CASE(2, 4, 4) FP6MI_CASE(2, 4, 8)
+        FP6MI_CASE(2, 5, 4) FP6MI_CASE(2, 5, 8) FP6MI_CASE(2, 6, 4) FP6MI_CASE(2, 7, 4) FP6MI_CASE(2, 8, 4)
 #undef FP6MI_CASE
     } else if (c.kind == 1) {
 #define FP6MI_CASE(NT, RT, WR, WK) \

@@ -26,7 +26,8 @@ INC_PATH = os.path.join(HERE, "csrc", "fp6mi_tuning.inc")
 
 # (kind, n_tiles, row_tiles, row_waves, k_waves); kind 0 = stream kernel (batch <= 16 per n_tile), 1 = tile kernel, 2 = wave-specialized tile kernel
 STREAM_SMALL = [(0, 1, rt, 1, wk) for rt in (1, 2, 3, 4, 5, 6, 7, 8) for wk in (4, 8, 16) if wk == 4 or (wk == 8 and rt <= 6) or rt <= 2]
-STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 3, 1, 4), (0, 2, 3, 1, 8), (0, 2, 4, 1, 4), (0, 2, 4, 1, 8)]   # two 16-column tiles per workgroup, batches 17..32
+STREAM_WIDE = [(0, 2, 1, 1, 8), (0, 2, 2, 1, 4), (0, 2, 3, 1, 4), (0, 2, 3, 1, 8), (0, 2, 4, 1, 4), (0, 2, 4, 1, 8), (0, 2, 5, 1, 4), (0, 2, 5, 1, 8),
+               (0, 2, 6, 1, 4), (0, 2, 7, 1, 4), (0, 2, 8, 1, 4)]   # two 16-column tiles per workgroup, batches 17..32
 TILE = [(1, 2, 1, 4, 4), (1, 2, 1, 2, 4), (1, 2, 2, 4, 1), (1, 2, 2, 4, 2), (1, 4, 1, 4, 2), (1, 4, 1, 8, 2), (1, 4, 2, 4, 2), (1, 4, 2, 8, 1),
         (1, 8, 2, 8, 1)]
 SPLITS = (1, 2, 3, 4, 6, 8)      # 3 and 6 fill 256 CUs where 80 or 40 row blocks leave a power of two short (M = 10240, 5120)
@@ -37,7 +38,7 @@ FORMAT_OF_BITS = {6: (3, 2), 5: (2, 2), 4: (2, 1)}   # the table is keyed by bit
 COMPILED_STREAM = [(0, nt, rt, 1, wk) for (nt, rt, wk) in
                    [(1, 1, 4), (1, 1, 8), (1, 1, 16), (1, 2, 4), (1, 2, 8), (1, 2, 16), (1, 3, 4), (1, 3, 8), (1, 4, 4), (1, 4, 8), (1, 5, 4),
                     (1, 5, 8), (1, 6, 4), (1, 6, 8), (1, 7, 4), (1, 8, 4), (2, 1, 4), (2, 1, 8), (2, 2, 4), (2, 2, 8), (2, 3, 4), (2, 3, 8),
-                    (2, 4, 4), (2, 4, 8)]]
+                    (2, 4, 4), (2, 4, 8), (2, 5, 4), (2, 5, 8), (2, 6, 4), (2, 7, 4), (2, 8, 4)]]
 COMPILED_TILE = [(1,) + c for c in
                  [(2, 1, 4, 4), (2, 2, 4, 4), (2, 2, 4, 2), (2, 2, 4, 1), (2, 4, 4, 1), (2, 4, 4, 2), (4, 2, 4, 2), (4, 2, 4, 1), (4, 4, 4, 1),
                   (4, 4, 2, 1), (4, 4, 2, 2), (8, 2, 4, 1), (8, 2, 2, 1), (4, 2, 8, 1), (4, 2, 8, 2), (2, 2, 8, 1), (2, 2, 8, 2), (8, 2, 8, 1),
