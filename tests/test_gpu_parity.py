@@ -709,6 +709,23 @@ def test_command_line_harness_suites(monkeypatch):
     assert len(rows) == 4 and all(r["max_rel_err_vs_fp32"] <= 1e-2 for r in rows) and buf.getvalue().count("speed-up") == 4
 
 
+def test_rules_give_a_cu_its_whole_share_of_row_tiles_in_one_workgroup():
+    """Far from every measured problem (K of a few hundred) the launch shape comes from the rules; for batches 5..16 they take
+    ceil(row tiles / 256 CUs) tiles per workgroup, which need not divide the row tiles.  Shapes and results are checked."""
+    E, M = 3, 2
+    L = _lib.lib()
+    shape = (ctypes.c_int * 5)()
+    for (OC, IC, N, want_rt) in [(10496, 512, 8, 3), (17664, 512, 12, 5), (21760, 448, 6, 6), (28160, 320, 9, 7)]:
+        assert L.fp6mi_launch_source(E, M, OC, N, IC, 1) == 2, "expected the rules to answer"
+        assert L.fp6mi_query_launch(E, M, OC, N, IC, 1, shape) == 0
+        assert shape[0] == 0 and shape[2] == want_rt and (OC // 16) % want_rt != 0, tuple(shape)
+        print("case rules", OC, IC, N, tuple(shape), flush=True)
+        raw, sc, x = synth.uniform_problem(9100 + N, OC, IC, N, E, M)
+        native, scd, xd = upload(raw, sc, x, E, M)
+        y = gemm_capi(E, M, native, scd, xd, OC)
+        check_close(y, oracle.gemm_f64(oracle.dequant(raw, sc, E, M), x), "rules %dx%d N=%d" % (OC, IC, N))
+
+
 @pytest.mark.parametrize("E,M", FORMATS)
 def test_random_shapes_through_the_automatic_launch_choice(E, M):
     """Forty seeded random problems per format -- rows in multiples of 256, columns in multiples of 64 (most of them not
