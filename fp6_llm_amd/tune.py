@@ -256,8 +256,10 @@ def emit(args):
         lines.append("{%d,%d,%d,%d,{%s}}," % (xb, OC // 256, IC // 64, BS, ",".join(cells)))
     with open(INC_PATH, "w") as f:
         f.write("\n".join(lines) + "\n")
+    note_path = os.path.join(os.path.dirname(os.path.abspath(__file__)), "tuning", "note.txt")   # what differs between the versions of the stamps
+    note = " ".join(open(note_path).read().split()) if os.path.exists(note_path) else ""
     with open(INC_PATH.replace(".inc", "_info.inc"), "w") as f:   # the same stamp as a string the library can report
-        f.write('"%d entries; %s"\n' % (len(rows), stamp_text.replace('"', "'")))
+        f.write('"%d entries; %s%s"\n' % (len(rows), stamp_text.replace('"', "'"), ("; " + note.replace('"', "'")) if note else ""))
     print("%d entries -> %s" % (len(rows), INC_PATH))
 
 
